@@ -3,7 +3,8 @@
 // token at sequence index p sees keys lo..p of its request, lo = max(0, p - window + 1) with
 // a window, else 0 (reference attention.py:336-402 for the mask, text.py:78 for the scale); with
 // a window it also sees the request's first `keep_first` keys, wherever the window stands.
-// Values may have another width (vd) than keys (hd).
+// Values may have another width (vd) than keys (hd).  With `sinks` (one float32 per query head) the
+// softmax's denominator also holds exp(sink): a place that has no key and no value and is not scaled.
 // Keys are walked in blocks of 64 by absolute index, so a token's result does not depend on
 // how its request was cut into steps or on what else is in the batch.
 #include "common.h"
@@ -15,7 +16,7 @@ __global__ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict
                                     const int* __restrict__ block_table, int table_width,
                                     const int* __restrict__ token_req, const int* __restrict__ token_seqpos,
                                     T* __restrict__ out, int nh, int nkv, int hd, int vd, int ps, int window,
-                                    int keep_first, float scale) {
+                                    int keep_first, float scale, const float* __restrict__ sinks) {
   __shared__ float sq[ATTN_MAX_HD];
   const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = token_req[n], p = token_seqpos[n];
@@ -68,6 +69,14 @@ __global__ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict
     }
     m = m_new;
   }
+  if (sinks) {
+    const float sk = sinks[h];
+    const float m_all = fmaxf(m, sk);
+    const float alpha = expf(m - m_all);
+    l = l * alpha + expf(sk - m_all);
+#pragma unroll
+    for (int i = 0; i < ATTN_MAX_HD / 64; ++i) acc[i] *= alpha;
+  }
   T* o = out + ((size_t)n * nh + h) * vd;
   const float inv = 1.0f / l;
 #pragma unroll
@@ -80,7 +89,7 @@ __global__ void attn_generic_kernel(const T* __restrict__ q, const T* __restrict
 extern "C" int qvl_attn_generic(const void* q, const void* kc, const void* vc, const void* block_table,
                                 int table_width, const void* token_req, const void* token_seqpos, void* out, int N,
                                 int nh, int nkv, int hd, int vd, int ps, int window, int keep_first, float scale,
-                                int dtype, hipStream_t stream) {
+                                const void* sinks, int dtype, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv || hd <= 0 || vd <= 0 || ps <= 0 || table_width <= 0 || keep_first < 0)
     return QVL_ERR_SHAPE;
@@ -89,11 +98,13 @@ extern "C" int qvl_attn_generic(const void* q, const void* kc, const void* vc, c
   if (dtype == 0)
     hipLaunchKernelGGL(attn_generic_kernel<float>, grid, dim3(64), 0, stream, (const float*)q, (const float*)kc,
                        (const float*)vc, (const int*)block_table, table_width, (const int*)token_req,
-                       (const int*)token_seqpos, (float*)out, nh, nkv, hd, vd, ps, window, keep_first, scale);
+                       (const int*)token_seqpos, (float*)out, nh, nkv, hd, vd, ps, window, keep_first, scale,
+                       (const float*)sinks);
   else if (dtype == 1)
     hipLaunchKernelGGL(attn_generic_kernel<bf16_t>, grid, dim3(64), 0, stream, (const bf16_t*)q, (const bf16_t*)kc,
                        (const bf16_t*)vc, (const int*)block_table, table_width, (const int*)token_req,
-                       (const int*)token_seqpos, (bf16_t*)out, nh, nkv, hd, vd, ps, window, keep_first, scale);
+                       (const int*)token_seqpos, (bf16_t*)out, nh, nkv, hd, vd, ps, window, keep_first, scale,
+                       (const float*)sinks);
   else
     return QVL_ERR_DTYPE;
   return qvl_launch_status();

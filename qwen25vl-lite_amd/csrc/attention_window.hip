@@ -1,5 +1,6 @@
 // Paged attention on the matrix cores for what the other matrix-core kernel does not take: a sliding
-// window that also keeps a request's first keys visible, and values of another width than keys.
+// window that also keeps a request's first keys visible, values of another width than keys, and a softmax
+// whose denominator holds one more term per query head, exp(sink), with no key and no value behind it.
 // bfloat16 storage, float32 scores, softmax and sums.  Compiled per key size HD and value size VD.
 //
 // A column is a (token, query head of one key/value head's group) pair; a tile has 16 of them.  A
@@ -51,6 +52,7 @@ struct WindowArgs {
   bf16_t* out;            // [N, nq, VD]
   int nq, nkv, ps, window, keep_first;
   float scale;
+  const float* sinks;     // [nq] float32, or null
 };
 
 // W: waves that share an entry's key blocks (1 or 4).  CT: column tiles of an entry, all carried by the
@@ -223,6 +225,14 @@ __global__ __launch_bounds__(256) void attn_window_kernel(WindowArgs a) {
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
     if (!valid[c]) continue;
+    if (a.sinks) {
+      const float sk = a.sinks[head[c]];
+      const float m_all = fmaxf(m[c], sk);
+      const float f = expf(m[c] - m_all);
+      l[c] = l[c] * f + expf(sk - m_all);
+#pragma unroll
+      for (int dt = 0; dt < NT; ++dt) acc[c][dt] *= f;
+    }
     const float inv = 1.0f / l[c];
     bf16_t* o = a.out + ((size_t)token[c] * a.nq + head[c]) * VD;
 #pragma unroll
@@ -254,7 +264,7 @@ extern "C" int qvl_attn_window_sizes(int* hd, int* vd) {
 extern "C" int qvl_attn_window(const void* q, const void* kc, const void* vc, const void* bt, int table_width,
                                const void* cu_q, const void* ctx_len, const void* tile_req, const void* tile_ct,
                                int num_tiles, void* out, int nq, int nkv, int ps, int window, int keep_first, float scale,
-                               int share, hipStream_t stream) {
+                               const void* sinks, int share, hipStream_t stream) {
   if (num_tiles <= 0) return QVL_OK;
   if (nq <= 0 || nkv <= 0 || nq % nkv || ps <= 0 || ps % 8 || table_width <= 0 || window < 0 || keep_first < 0)
     return QVL_ERR_SHAPE;
@@ -265,6 +275,7 @@ extern "C" int qvl_attn_window(const void* q, const void* kc, const void* vc, co
   a.table_width = table_width; a.cu_q = (const int*)cu_q; a.ctx_len = (const int*)ctx_len;
   a.tile_req = (const int*)tile_req; a.tile_ct = (const int*)tile_ct; a.num_tiles = num_tiles; a.out = (bf16_t*)out;
   a.nq = nq; a.nkv = nkv; a.ps = ps; a.window = window; a.keep_first = keep_first; a.scale = scale;
+  a.sinks = (const float*)sinks;
   if (share) hipLaunchKernelGGL((attn_window_kernel<4, 1>), dim3(num_tiles, nkv), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL((attn_window_kernel<1, WIDE_CT>), dim3((num_tiles + 3) / 4, nkv), dim3(256), 0, stream, a);
   return qvl_launch_status();

@@ -166,6 +166,7 @@ extern "C" int qvl_moe_sort(const void* ids, void* sorted, void* offsets, int P,
 //   plain:  out[p, c] = in . W[e, c, :]
 //   gated:  g = min(in . W[e, c, :], limit), u = clamp(in . W[e, R + c, :], -limit, limit)  (no clamps if limit <= 0)
 //           out[p, c] = g * sigmoid(alpha g) * (u + shift)            (W[e] holds R gate rows, then R up rows)
+//   plain with act 1:  out[p, c] = max(in . W[e, c, :], 0)^2
 // Any sizes and both storage types: one wave per output value, lanes split K (the sum's order is fixed).
 // ---------------------------------------------------------------------------------------
 struct ExpertArgs {
@@ -176,6 +177,7 @@ struct ExpertArgs {
   const int* offsets;
   void* out;            // [P, R]
   int P, E, R, K, div, gated;
+  int act;              // on a plain product's values: 0 none, 1 the square of relu
   float alpha, limit, shift;
 };
 
@@ -185,6 +187,14 @@ __device__ __forceinline__ float gated_value(float g, float u, float alpha, floa
     u = fminf(fmaxf(u, -limit), limit);
   }
   return g * sigmoid_f(alpha * g) * (u + shift);
+}
+
+__device__ __forceinline__ float plain_value(float v, int act) {
+  if (act == 1) {
+    v = fmaxf(v, 0.f);
+    v *= v;
+  }
+  return v;
 }
 
 __device__ __forceinline__ int expert_of(const int* offsets, int E, int i) {
@@ -211,6 +221,8 @@ __global__ __launch_bounds__(256) void moe_rows_kernel(ExpertArgs a) {
       for (int k = lane; k < a.K; k += 64) u += ldf<T>(xr + k) * ldf<T>(wu + k);
       u = wave_sum(u);
       g = gated_value(g, u, a.alpha, a.limit, a.shift);
+    } else {
+      g = plain_value(g, a.act);
     }
     if (lane == 0) stf<TO>((TO*)a.out + (size_t)p * a.R + c, g);
   }
@@ -289,6 +301,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
       if (c0 + 4 * lg + j >= a.R) break;
       float v = accg[t][j];
       if (a.gated) v = gated_value(v, accu[t][j], a.alpha, a.limit, a.shift);
+      else v = plain_value(v, a.act);
       stf<TO>(o + j, v);
     }
   }
@@ -459,6 +472,7 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
         if (c + j >= a.R) break;
         float v = acc[n][m][j];
         if (GATED) v = gated_value(v, acc[n + NW / 2][m][j], a.alpha, a.limit, a.shift);
+        else v = plain_value(v, a.act);
         stf<TO>(o + c + j, v);
       }
     }
@@ -606,6 +620,7 @@ __global__ __launch_bounds__(256) void moe_stream_kernel(ExpertArgs a, int tiles
         if (c + j >= a.R) break;
         float v = acc[n][m][j];
         if (GATED) v = gated_value(v, acc[n + ST_NW / 2][m][j], a.alpha, a.limit, a.shift);
+        else v = plain_value(v, a.act);
         stf<TO>(o + c + j, v);
       }
     }
@@ -617,12 +632,13 @@ __global__ __launch_bounds__(256) void moe_stream_kernel(ExpertArgs a, int tiles
 // 16-byte boundaries; `big_tiles` asks for the kernel with tiles of 128 pairs through LDS (many pairs an expert).
 extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const void* w, const void* sorted,
                                const void* offsets, void* out, int out_dtype, int P, int E, int R, int K, int div,
-                               int gated, float alpha, float limit, float shift, int big_tiles, hipStream_t stream) {
+                               int gated, float alpha, float limit, float shift, int act, int big_tiles,
+                               hipStream_t stream) {
   if (P <= 0) return QVL_OK;
   if (E <= 0 || R <= 0 || K <= 0 || div <= 0 || ldx < K || !x || !w || !sorted || !offsets || !out) return QVL_ERR_SHAPE;
   ExpertArgs a;
   a.x = x; a.ldx = ldx; a.w = w; a.sorted = (const int*)sorted; a.offsets = (const int*)offsets; a.out = out;
-  a.P = P; a.E = E; a.R = R; a.K = K; a.div = div; a.gated = gated; a.alpha = alpha; a.limit = limit; a.shift = shift;
+  a.P = P; a.E = E; a.R = R; a.K = K; a.div = div; a.gated = gated; a.act = gated ? 0 : act; a.alpha = alpha; a.limit = limit; a.shift = shift;
   if (x_dtype == 1 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0) {
     if (out_dtype != 0 && out_dtype != 1) return QVL_ERR_DTYPE;
 #ifndef MOE_NO_STREAM

@@ -1,0 +1,77 @@
+// A short causal convolution over time on every channel, added to its input:
+//   out[t, c] = x[t, c] + sum_j w[c, j] * x[t - taps + 1 + j, c],   j = 0 .. taps - 1
+// over the tokens of one request; inputs before the request's first token are zeros.  The last taps - 1
+// inputs of a request are its state (float32 [slots, taps - 1, C], oldest first), read by the first tokens
+// of the request's next run and replaced at the end of this one.  x is the float32 residual; the result is
+// written in the run's storage type.
+//
+// Grid (N + R, channel blocks).  Rows below N are tokens: a token that stands at least taps - 1 tokens into
+// its run reads only x.  The last R rows are requests: the thread of a channel forms the outputs of the
+// run's first taps - 1 tokens from the old state and then writes the new one, so nobody else reads or
+// writes that channel of the slot in this launch.
+#include "common.h"
+
+template <typename TO>
+__global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                         float* __restrict__ state, const int* __restrict__ cu_q,
+                                                         const int* __restrict__ req_slots,
+                                                         const int* __restrict__ token_req, TO* __restrict__ out, int N,
+                                                         int C, int taps) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const float* wc = w + (size_t)c * taps;
+  const int keep = taps - 1;
+  if ((int)blockIdx.x < N) {
+    const int t = blockIdx.x;
+    const int i = t - cu_q[token_req[t]];
+    if (i < keep) return;                       // the request's row forms it from the state
+    float acc = x[(size_t)t * C + c];
+    for (int j = 0; j < taps; ++j) acc += wc[j] * x[(size_t)(t - keep + j) * C + c];
+    stf<TO>(out + (size_t)t * C + c, acc);
+    return;
+  }
+  const int r = blockIdx.x - N;
+  const int begin = cu_q[r], n = cu_q[r + 1] - begin;
+  if (n <= 0) return;
+  float* st = state + (size_t)req_slots[r] * keep * C + c;      // st[k * C]: input number k of the kept ones
+  const int first = n < keep ? n : keep;
+  for (int i = 0; i < first; ++i) {
+    float acc = x[(size_t)(begin + i) * C + c];
+    for (int j = 0; j < taps; ++j) {
+      const int src = i - keep + j;             // index into this run; negative: the kept inputs
+      const float v = src >= 0 ? x[(size_t)(begin + src) * C + c] : st[(size_t)(keep + src) * C];
+      acc += wc[j] * v;
+    }
+    stf<TO>(out + (size_t)(begin + i) * C + c, acc);
+  }
+  // the last `keep` inputs of (kept inputs, this run); entry k comes from a place behind k, so ascending order
+  // never reads what it has overwritten
+  for (int k = 0; k < keep; ++k) {
+    const int at = n + k;                       // index into (kept inputs, this run)
+    st[(size_t)k * C] = at < keep ? st[(size_t)at * C] : x[(size_t)(begin + at - keep) * C + c];
+  }
+}
+
+// x float32 [N, C]; w float32 [C, taps]; state float32 [slots, taps - 1, C] (unused with taps == 1);
+// cu_q [R + 1], req_slots [R], token_req [N] int32; out [N, C] of out_dtype (0 float32, 1 bfloat16).
+extern "C" int qvl_short_conv(const void* x, const void* w, void* state, const void* cu_q, const void* req_slots,
+                              const void* token_req, void* out, int out_dtype, int N, int R, int C, int taps,
+                              hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (R <= 0 || C <= 0 || taps < 1 || !x || !w || !out || !cu_q || !token_req) return QVL_ERR_SHAPE;
+  if (taps > 1 && (!state || !req_slots)) return QVL_ERR_SHAPE;
+  const long long rows = (long long)N + (taps > 1 ? R : 0);
+  if (rows > 0x7fffffffll || (C + 255) / 256 > 65535) return QVL_ERR_LIMIT;
+  const dim3 grid((unsigned)rows, (C + 255) / 256);
+  if (out_dtype == 0)
+    hipLaunchKernelGGL(short_conv_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (const float*)w,
+                       (float*)state, (const int*)cu_q, (const int*)req_slots, (const int*)token_req, (float*)out, N, C,
+                       taps);
+  else if (out_dtype == 1)
+    hipLaunchKernelGGL(short_conv_kernel<bf16_t>, grid, dim3(256), 0, stream, (const float*)x, (const float*)w,
+                       (float*)state, (const int*)cu_q, (const int*)req_slots, (const int*)token_req, (bf16_t*)out, N, C,
+                       taps);
+  else
+    return QVL_ERR_DTYPE;
+  return qvl_launch_status();
+}

@@ -28,11 +28,12 @@ def _prefix_of(name: str) -> str:
     return name[:name.rfind(".") + 1]
 
 
-def _mixers_of(block: Part, prefix: str = "") -> List[Tuple[str, Mixer]]:
-    """Every mixer inside a block, however deep, with its dotted sub-part name."""
-    found: List[Tuple[str, Mixer]] = []
+def _mixers_of(block: Part, prefix: str = "") -> List[Tuple[str, Part]]:
+    """Every mixer inside a block, however deep, and every other part that keeps a cache or a per-request
+    state (a short convolution), with its dotted sub-part name."""
+    found: List[Tuple[str, Part]] = []
     for name, sub in block.sub_parts().items():
-        if isinstance(sub, Mixer):
+        if isinstance(sub, Mixer) or sub.state_need() is not None or sub.cache_need() is not None:
             found.append((prefix + name, sub))
         else:
             found.extend(_mixers_of(sub, f"{prefix}{name}."))

@@ -12,15 +12,17 @@ __all__ = ["paged_attention"]
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
-                    step, num_q_heads: int, window: Optional[int], scale: float, keep_first: int = 0) -> torch.Tensor:
+                    step, num_q_heads: int, window: Optional[int], scale: float, keep_first: int = 0,
+                    sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages.
 
-    bfloat16 with a head size in steps of 16 runs on the matrix cores; everything else
-    bfloat16 with a window that keeps the first keys, or values of another width than the keys, has a
+    bfloat16 with a head size in steps of 16 runs on the matrix cores;
+    bfloat16 with a window that keeps the first keys, values of another width than the keys, or ``sinks``
+    (float32 ``[heads]``: one more term ``exp(sink)`` in each head's softmax denominator) has a
     matrix-core kernel of its own; everything else (float32, other head sizes) runs through the
     float32-arithmetic kernel.
     """
-    plain = not (window and keep_first) and v_cache.shape[2] == k_cache.shape[3]
+    plain = not (window and keep_first) and v_cache.shape[2] == k_cache.shape[3] and sinks is None
     if q.dtype == torch.bfloat16 and plain:
         from . import attention_mfma
         out = attention_mfma.try_attention(q, k_cache, v_cache, block_table, step, num_q_heads, window, scale)
@@ -29,8 +31,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     elif q.dtype == torch.bfloat16:
         from . import attention_window
         out = attention_window.try_attention(q, k_cache, v_cache, block_table, step, num_q_heads, window, keep_first,
-                                             scale)
+                                             scale, sinks=sinks)
         if out is not None:
             return out
     return kernels.paged_attention_generic(q, k_cache, v_cache, block_table, step.token_req, step.token_seqpos,
-                                           num_q_heads, window, scale, keep_first=keep_first)
+                                           num_q_heads, window, scale, keep_first=keep_first, sinks=sinks)

@@ -1,5 +1,6 @@
-"""Dispatch to the matrix-core attention for windows that keep a request's first keys and for values
-of another width than keys (bfloat16; key sizes in steps of 8 up to 256, value sizes up to 256).
+"""Dispatch to the matrix-core attention for windows that keep a request's first keys, for values
+of another width than keys and for a softmax with one more term per head in its denominator
+(bfloat16; key sizes in steps of 8 up to 256, value sizes up to 256).
 
 The kernel is compiled per (key size, value size) at its first use.  Tiles are the other matrix-core
 kernel's: 16 columns, a column being a (token, query head of one key/value group) pair.
@@ -28,7 +29,8 @@ def supports(head_dim: int, value_dim: int, page_size: int, dtype: torch.dtype) 
 
 
 def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, window: Optional[int], keep_first: int,
-                  scale: float, share: Optional[bool] = None) -> Optional[torch.Tensor]:
+                  scale: float, share: Optional[bool] = None, sinks: Optional[torch.Tensor] = None
+                  ) -> Optional[torch.Tensor]:
     """The attention through this kernel, or None if it does not take the shape.  ``share`` (tests):
     whether the waves of a block share a tile, else chosen by the number of tiles."""
     pages, nkv, ps, hd = k_cache.shape
@@ -42,6 +44,8 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
           and block_table.shape[0] == step.num_reqs, "block_table must be int32 [R, width]")
     _need(nq % nkv == 0, "query heads must be a multiple of key/value heads")
+    _need(sinks is None or (sinks.is_cuda and sinks.dtype == torch.float32 and sinks.shape == (nq,)
+                            and sinks.is_contiguous()), "sinks must be float32 [nq] on the GPU")
     group = nq // nkv
     defines = {"HD": hd, "VD": vd}
     tile_req, tile_ct, num_tiles = _step_tiles(step, group, 1, q.device)
@@ -56,11 +60,11 @@ def try_attention(q, k_cache, v_cache, block_table, step, num_q_heads: int, wind
         tile_req, tile_ct, num_tiles = _step_tiles(step, group, wide, q.device)
     out = torch.empty((n, nq * vd), dtype=q.dtype, device=q.device)
     fn = _fn("attention_window", "qvl_attn_window",
-             [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 5 + [_c_float, _c_int, _c_ptr],
+             [_c_ptr] * 4 + [_c_int] + [_c_ptr] * 4 + [_c_int, _c_ptr] + [_c_int] * 5 + [_c_float, _c_ptr, _c_int, _c_ptr],
              defines)
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(cu_q),
               _ptr(step.ctx_len), _ptr(tile_req), _ptr(tile_ct), num_tiles, _ptr(out), nq, nkv, ps, int(window or 0),
-              int(keep_first) if window else 0, float(scale), int(bool(share)), _stream()),
+              int(keep_first) if window else 0, float(scale), _ptr(sinks), int(bool(share)), _stream()),
            "paged_attention (matrix cores, window with kept keys)")
     taken["window with kept keys, " + ("shared tiles" if share else "a wave per tile")] += 1
     return out

@@ -21,6 +21,9 @@ LIBRARIES = [
     ("peaks", {}),
     ("gated", {}),
     ("moe", {}),
+    ("rownorm", {}),
+    ("short_conv", {}),
+    ("latent", {}),
     # the linear-attention kernels are compiled per key size (the sizes the tests and the benchmark
     # use; any other size up to 512 is compiled at its first use)
     *[("linear_attention", {"LA_DIM": d}) for d in (5, 6, 8, 12, 16, 20, 32, 64, 128, 320)],

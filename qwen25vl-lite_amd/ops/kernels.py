@@ -241,15 +241,17 @@ def copy_pages(cache: torch.Tensor, src: Sequence[int], dst: Sequence[int]) -> N
 def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                             block_table: torch.Tensor, token_req: torch.Tensor, token_seqpos: torch.Tensor,
                             num_q_heads: int, window: Optional[int], scale: float,
-                            out: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
+                            out: Optional[torch.Tensor] = None, keep_first: int = 0,
+                            sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of every token over its request's pages; any head size, float32 arithmetic.
 
     ``q`` is ``[N, nq hd]``; token ``n`` belongs to row ``token_req[n]`` of ``block_table`` and
     sits at sequence index ``token_seqpos[n]``; it sees keys ``max(0, p - window + 1) .. p`` and,
     with a window, the first ``keep_first`` keys of its request.  The result is ``[N, nq vd]``,
-    ``vd`` being the value width of ``v_cache [pages, nkv, vd, page_size]``.
+    ``vd`` being the value width of ``v_cache [pages, nkv, vd, page_size]``.  ``sinks`` (float32 ``[nq]``): the
+    softmax's denominator of head ``h`` also holds ``exp(sinks[h])``, a term with no key and no value.
     """
-    _dev(q, k_cache, v_cache, block_table, token_req, token_seqpos, out)
+    _dev(q, k_cache, v_cache, block_table, token_req, token_seqpos, out, sinks)
     n = q.shape[0]
     nq = int(num_q_heads)
     _need(k_cache.dim() == 4 and k_cache.is_contiguous() and v_cache.is_contiguous(), "cache must be contiguous")
@@ -267,12 +269,14 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         out = torch.empty((n, nq * vd), dtype=q.dtype, device=q.device)
     _need(out.shape == (n, nq * vd) and out.dtype == q.dtype and out.is_contiguous(), "out must be [N, nq vd]")
     _need(keep_first >= 0, "keep_first cannot be negative")
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.shape == (nq,) and sinks.is_contiguous()),
+          "sinks must be float32 [nq]")
     fn = _fn("attention_generic", "qvl_attn_generic",
              [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
-              _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_int, _c_ptr])
     _check(fn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(token_req),
               _ptr(token_seqpos), _ptr(out), n, nq, nkv, hd, vd, ps, int(window or 0),
-              int(keep_first) if window else 0, float(scale), dtype_code(q.dtype), _stream()),
+              int(keep_first) if window else 0, float(scale), _ptr(sinks), dtype_code(q.dtype), _stream()),
            "paged_attention_generic")
     return out
 

@@ -30,25 +30,30 @@ CHUNKED_FROM = 128    # a step whose longest run has this many tokens or more is
 def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_heads: int, dim: int, vdim: int,
                  state: torch.Tensor, cu_q: torch.Tensor, req_slots: torch.Tensor, *,
                  head_decay: Optional[torch.Tensor] = None, z: Optional[torch.Tensor] = None, tau: float = 1.0,
-                 silu: bool = False, q_scale: float = 1.0, groups: int = 1,
-                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 silu=False, q_scale: float = 1.0, groups: int = 1, out: Optional[torch.Tensor] = None,
+                 lower: Optional[torch.Tensor] = None, z_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Run every request's tokens of the step through the recurrence, from and into ``state``.
 
     ``proj [N, cols]`` (float32 or bfloat16) holds, per token, ``heads * dim`` query columns from
     ``q_off``, as many key columns from ``k_off`` and ``heads * vdim`` value columns from ``v_off``;
-    ``silu`` applies the activation to all three as they are read, ``q_scale`` scales the queries.
+    ``silu`` applies the activation as they are read (True: to all three; or a string naming which, e.g.
+    ``"q"``), ``q_scale`` scales the queries.
     The decay is ``head_decay [heads]`` (float32, one constant per head) or, per token and key
-    channel, ``sigmoid(z)^(1/tau)`` for float32 ``z [N, heads * dim]``.  ``cu_q [R + 1]`` bounds each
+    channel, ``sigmoid(z)^(1/tau)`` for float32 ``z [N, heads * dim]``, or, with ``lower`` (float32
+    ``[heads * dim]``, and ``z_bias`` of the same shape or None), the floored forget gate
+    ``lower + (1 - lower) sigmoid(z + z_bias)``, whose complement ``1 - decay`` is then the key (no key
+    columns are read).  ``cu_q [R + 1]`` bounds each
     request's run of tokens, ``req_slots [R]`` names its row of ``state``.  Returns float32
     ``[groups, N, heads * vdim]``: with ``groups`` above 1 (2, 4 or 8; the key size must be a multiple
     of four times it) the key channels are cut into that many groups with blocks of their own, and the
     output is the sum of the slabs (see :func:`scan_groups`)."""
-    _dev(proj, state, cu_q, req_slots, head_decay, z)
+    _dev(proj, state, cu_q, req_slots, head_decay, z, lower, z_bias)
     h, d, v = int(num_heads), int(dim), int(vdim)
     n = proj.shape[0]
     _need(1 <= d <= MAX_KEY_SIZE, f"key sizes up to {MAX_KEY_SIZE} are built")
     _need(proj.dim() == 2 and proj.stride(1) == 1, "proj must be [N, cols] with contiguous rows")
-    for off, width in ((q_off, h * d), (k_off, h * d), (v_off, h * v)):
+    _check_forget(lower, z_bias, z, h * d)
+    for off, width in ((q_off, h * d), (q_off if lower is not None else k_off, h * d), (v_off, h * v)):
         _need(0 <= off and off + width <= proj.shape[1], "q, k or v columns lie outside proj")
     _need(state.dtype == torch.float32 and state.dim() == 4 and tuple(state.shape[1:]) == (h, d, v)
           and state.is_contiguous(), "state must be contiguous float32 [slots, heads, dim, vdim]")
@@ -73,11 +78,34 @@ def decayed_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
           "out must be contiguous float32 [groups, N, heads vdim]")
     fn = _fn("linear_attention", "qvl_la_scan",
              [_c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr, _c_ptr, _c_ptr,
-              _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr], {"LA_DIM": d})
+              _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr],
+             {"LA_DIM": d})
     _check(fn(_ptr(proj), proj.stride(0), int(q_off), int(k_off), int(v_off), dtype_code(proj.dtype),
-              _ptr(head_decay), _ptr(z), zstride, 1.0 / float(tau), _ptr(state), _ptr(cu_q), _ptr(req_slots),
-              _ptr(out), out.stride(0), int(groups), r, h, d, v, int(silu), float(q_scale), _stream()), "decayed_scan")
+              _ptr(head_decay), _ptr(z), zstride, 1.0 / float(tau), _ptr(lower), _ptr(z_bias), _ptr(state), _ptr(cu_q),
+              _ptr(req_slots), _ptr(out), out.stride(0), int(groups), r, h, d, v, silu_mask(silu), float(q_scale),
+              _stream()), "decayed_scan")
     return out
+
+
+def silu_mask(silu) -> int:
+    """Which of q, k and v pass through silu as they are read, as the kernels' bit mask (1 q, 2 k, 4 v): True means
+    all three, False or None none, a string names them (``"q"``, ``"qk"``, ...)."""
+    if silu is True:
+        return 7
+    if not silu:
+        return 0
+    _need(set(silu) <= set("qkv"), "silu names some of q, k and v")
+    return sum(bit for name, bit in (("q", 1), ("k", 2), ("v", 4)) if name in silu)
+
+
+def _check_forget(lower, z_bias, z, width: int) -> None:
+    if lower is None:
+        _need(z_bias is None, "a bias on z belongs to the floored forget gate")
+        return
+    _need(z is not None, "the floored forget gate needs z")
+    for t in (lower, z_bias):
+        _need(t is None or (t.dtype == torch.float32 and t.shape == (width,) and t.is_contiguous()),
+              "lower and z_bias must be float32 [heads dim]")
 
 
 def scan_groups(num_reqs: int, max_run: int, num_heads: int, dim: int, vdim: int, device=None) -> int:
@@ -126,7 +154,8 @@ def plan_chunks(cu_q_host: Sequence[int], device, chunk_len: int = CHUNK) -> Chu
 def chunked_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_heads: int, dim: int, vdim: int,
                  state: torch.Tensor, plan: ChunkPlan, req_slots: torch.Tensor, *,
                  head_decay: Optional[torch.Tensor] = None, z: Optional[torch.Tensor] = None, tau: float = 1.0,
-                 silu: bool = False, q_scale: float = 1.0) -> torch.Tensor:
+                 silu=False, q_scale: float = 1.0, lower: Optional[torch.Tensor] = None,
+                 z_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """:func:`decayed_scan` for steps with long runs: the chunks of ``plan`` are scanned side by side
     from zero states, the states are carried from chunk to chunk, and what the state before a chunk
     adds to the chunk's outputs is one float32 matrix product per (chunk, head), ``(q_t P_t) S``
@@ -140,16 +169,16 @@ def chunked_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, num_hea
     groups = scan_groups(nch, clen, h, d, v, proj.device)
     out = torch.empty((groups + 1, n, h * v), dtype=torch.float32, device=proj.device)
     decayed_scan(proj, q_off, k_off, v_off, h, d, v, scratch, plan.chunk_cu, plan.chunk_rows, head_decay=head_decay,
-                 z=z, tau=tau, silu=silu, q_scale=q_scale, groups=groups, out=out[:groups])
+                 z=z, tau=tau, silu=silu, q_scale=q_scale, groups=groups, out=out[:groups], lower=lower, z_bias=z_bias)
     qp = torch.zeros((nch, h, clen, d), dtype=torch.float32, device=proj.device)
     last = torch.empty((nch, h, d), dtype=torch.float32, device=proj.device)
     defines = {"LA_DIM": d}
     fn = _fn("linear_attention", "qvl_la_prefix",
-             [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
-              _c_int, _c_int, _c_int, _c_float, _c_ptr], defines)
+             [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ll, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+              _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr], defines)
     _check(fn(_ptr(proj), proj.stride(0), int(q_off), dtype_code(proj.dtype), _ptr(head_decay), _ptr(z),
-              z.stride(0) if z is not None else 0, 1.0 / float(tau), _ptr(plan.chunk_cu), _ptr(qp), _ptr(last), nch, h,
-              d, clen, int(silu), float(q_scale), _stream()), "chunk prefix")
+              z.stride(0) if z is not None else 0, 1.0 / float(tau), _ptr(lower), _ptr(z_bias), _ptr(plan.chunk_cu),
+              _ptr(qp), _ptr(last), nch, h, d, clen, silu_mask(silu), float(q_scale), _stream()), "chunk prefix")
     r = req_slots.shape[0]
     _need(plan.req_first.shape[0] == r + 1, "the chunk plan belongs to another step")
     fn = _fn("linear_attention", "qvl_la_carry", [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,

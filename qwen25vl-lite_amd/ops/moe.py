@@ -19,6 +19,7 @@ __all__ = ["route", "sort_pairs", "expert_products", "combine", "SCORE_FUNCTIONS
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 SCORE_FUNCTIONS = {"sigmoid": 0, "softmax": 1}
+PLAIN_ACTS = {None: 0, "relu2": 1}
 # from this many pairs per expert on (on average) the matrix-core kernels with tiles of 128 pairs through LDS run
 BIG_TILE_PAIRS = 32
 
@@ -61,19 +62,21 @@ def sort_pairs(ids: torch.Tensor, num_experts: int) -> Tuple[torch.Tensor, torch
 
 
 def expert_products(x: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, offsets: torch.Tensor, pairs: int,
-                    div: int, out_dtype: torch.dtype, gated: Optional[Tuple[float, Optional[float], float]] = None
-                    ) -> torch.Tensor:
+                    div: int, out_dtype: torch.dtype, gated: Optional[Tuple[float, Optional[float], float]] = None,
+                    act: Optional[str] = None) -> torch.Tensor:
     """``out[p] = x[p // div] @ weight[e(p)].T`` for every pair ``p``, ``e(p)`` the expert whose range
     of ``order`` holds it; ``weight`` is ``[E, R, K]``.  With ``gated = (alpha, limit, shift)``,
     ``weight`` is ``[E, 2 R, K]`` (R gate rows, then R up rows) and
     ``out[p] = g sigmoid(alpha g) (u + shift)`` with ``g`` capped at ``limit`` and ``u`` clamped to
-    ``[-limit, limit]`` (``limit`` None: no clamps).  Returns ``[pairs, R]`` in ``out_dtype``."""
+    ``[-limit, limit]`` (``limit`` None: no clamps).  Without ``gated``, ``act`` ``"relu2"`` squares the positive
+    part of every value of the product.  Returns ``[pairs, R]`` in ``out_dtype``."""
     _dev(x, weight, order, offsets)
     _need(weight.dim() == 3 and weight.is_contiguous() and x.dim() == 2 and x.stride(1) == 1
           and x.dtype == weight.dtype and x.shape[1] == weight.shape[2], "x [M, K] and weight [E, rows, K] of one dtype")
     e, rows_w, k = weight.shape
     r = rows_w // 2 if gated else rows_w
     _need(not gated or rows_w % 2 == 0, "gate and up rows come in equal numbers")
+    _need(act in PLAIN_ACTS and not (gated and act), "a plain product's activation is None or 'relu2'")
     _need(order.dtype == torch.int32 and order.shape == (pairs,) and offsets.dtype == torch.int32
           and offsets.shape == (e + 1,), "order must be int32 [pairs], offsets int32 [E + 1]")
     _need(pairs <= x.shape[0] * div, "a pair's row lies outside x")
@@ -82,10 +85,11 @@ def expert_products(x: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, 
     out = torch.empty((pairs, r), dtype=out_dtype, device=x.device)
     alpha, limit, shift = gated if gated else (1.0, None, 0.0)
     fn = _fn("moe", "qvl_moe_experts", [_c_ptr, _c_ll, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _c_ptr])
+                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _c_int,
+                                        _c_ptr])
     _check(fn(_ptr(x), x.stride(0), dtype_code(x.dtype), _ptr(weight), _ptr(order), _ptr(offsets), _ptr(out),
               dtype_code(out_dtype), int(pairs), e, r, k, int(div), int(bool(gated)), float(alpha), float(limit or 0.0),
-              float(shift), int(pairs >= BIG_TILE_PAIRS * e), _stream()), "moe experts")
+              float(shift), PLAIN_ACTS[act], int(pairs >= BIG_TILE_PAIRS * e), _stream()), "moe experts")
     return out
 
 

@@ -19,6 +19,8 @@ Kinds of parts and what each must provide:
 * ``PositionEncoding``: ``rotary_tables(head_dim, device)`` gives the per-frequency inverse
   frequencies and the row of the position tensor each frequency reads.
 * ``Block``: ``forward(stream, step, slot)`` arranges two norms, a mixer and a feed-forward.
+* ``Filter``: ``forward(h, step, slot) -> x``: what a sublayer reads, made from the float32 residual (a
+  short convolution over time); it may keep a per-request state like a mixer.
 
 New kinds are added with :func:`register_part` and named in a model's layer specs.
 """
@@ -32,7 +34,7 @@ import torch
 
 __all__ = [
     "ParamSpec", "PartSpec", "CacheNeed", "StateNeed", "LayerSlot", "GroupStep", "StepContext", "ResidualStream",
-    "Part", "Norm", "Mixer", "FeedForward", "PositionEncoding", "Block", "register_part", "build_part",
+    "Part", "Norm", "Mixer", "FeedForward", "Filter", "PositionEncoding", "Block", "register_part", "build_part",
     "known_parts", "Embedding", "Head",
 ]
 
@@ -43,7 +45,8 @@ class ParamSpec:
     ``"matrix"`` and ``"table"`` in the run dtype (bfloat16 or float32), ``"vector"`` in
     float32 (norm weights, biases: they enter float32 arithmetic), ``"int"`` as int32.
     ``init`` says how the random-weights mode draws it: ``"normal"`` N(0, std),
-    ``"around_one"`` 1 + N(0, std) (a gain), ``"zeros"``, ``"ones"``."""
+    ``"around_one"`` 1 + N(0, std) (a gain), ``"zeros"``, ``"ones"``, ``"unit_interval"`` uniform on [0, 1)
+    (a floor of a gate)."""
 
     shape: Tuple[int, ...]
     role: str = "matrix"
@@ -176,6 +179,15 @@ class Part:
     def sub_parts(self) -> Dict[str, "Part"]:
         return {}
 
+    def cache_need(self) -> Optional[CacheNeed]:
+        """Keys and values this part keeps per token in pages, or None."""
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        """A state of fixed size this part keeps per request, or None.  A part with either need gets a
+        :class:`LayerSlot` of its own for every entry of the run list that names its layer."""
+        return None
+
 
 class Norm(Part):
     def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
@@ -185,18 +197,21 @@ class Norm(Part):
 
 
 class Mixer(Part):
-    def cache_need(self) -> Optional[CacheNeed]:
-        return None
-
-    def state_need(self) -> Optional[StateNeed]:
-        return None
-
     def forward(self, x: torch.Tensor, step: StepContext, slot: LayerSlot) -> torch.Tensor:
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def forward(self, x: torch.Tensor, step: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Filter(Part):
+    """A transform of the float32 residual's rows on their way into a sublayer (a short convolution over
+    time); it may keep a state per request."""
+
+    def forward(self, h: torch.Tensor, step: StepContext, slot: LayerSlot) -> torch.Tensor:
+        """float32 ``[N, hidden]`` -> ``[N, hidden]`` in the run dtype."""
         raise NotImplementedError
 
 
@@ -241,7 +256,7 @@ class Head(Part):
 
 
 _REGISTRY: Dict[str, Dict[str, Callable[..., Part]]] = {
-    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
+    "norm": {}, "mixer": {}, "ffn": {}, "position": {}, "block": {}, "embedding": {}, "head": {}, "filter": {},
 }
 
 

@@ -4,9 +4,11 @@ from __future__ import annotations
 
 from typing import Dict, Optional
 
+import torch
+
 from .base import Block, LayerSlot, Part, PartSpec, ResidualStream, StepContext, build_part, register_part
 
-__all__ = ["PreNormBlock", "ParallelBlock", "SandwichBlock"]
+__all__ = ["PreNormBlock", "ParallelBlock", "SandwichBlock", "PostNormBlock"]
 
 
 class PreNormBlock(Block):
@@ -133,6 +135,73 @@ class SandwichBlock(Block):
         return stream
 
 
+class PostNormBlock(Block):
+    """``h += norm1(mixer(f(h))); h += norm2(ffn(h))``: the sublayers read the residual sum itself and the
+    norm stands on each sublayer's output only; ``f`` is an optional filter on what the mixer reads (a short
+    convolution over time with a state per request).
+
+    params: ``mixer``, ``norm1`` (:class:`PartSpec` each; the norm must offer ``add_normed``, as the layer
+    norm does), ``ffn`` and ``norm2`` (or ``ffn`` None for a layer without a feed-forward, whose ``norm2`` is
+    then not built), ``filter`` (a :class:`PartSpec` of category ``filter``, or None) and ``names``, the
+    checkpoint sub-name of each.  The sum stays float32; a sublayer is handed its rounding to the run dtype.
+    """
+
+    graph_safe = True
+
+    def __init__(self, params, dtype, device):
+        super().__init__(dtype, device)
+        self.names: Dict[str, str] = dict(params["names"])
+        self.mixer = build_part("mixer", params["mixer"], dtype, device)
+        self.norm1 = build_part("norm", params["norm1"], dtype, device)
+        self.filter: Optional[Part] = None
+        if params.get("filter") is not None:
+            self.filter = build_part("filter", params["filter"], dtype, device)
+        self.ffn: Optional[Part] = None
+        self.norm2: Optional[Part] = None
+        if params.get("ffn") is not None:
+            self.ffn = build_part("ffn", params["ffn"], dtype, device)
+            self.norm2 = build_part("norm", params["norm2"], dtype, device)
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not hasattr(norm, "add_normed"):
+                raise ValueError("the norm behind a sublayer must be able to add its result into the sum")
+
+    def sub_parts(self) -> Dict[str, Part]:
+        # the mixer first: an entry's own slot is its first part's
+        parts = {self.names["mixer"]: self.mixer, self.names["norm1"]: self.norm1}
+        if self.filter is not None:
+            parts[self.names["filter"]] = self.filter
+        if self.ffn is not None:
+            parts.update({self.names["ffn"]: self.ffn, self.names["norm2"]: self.norm2})
+        return parts
+
+    def _rounded(self, h):
+        return h if self.dtype == h.dtype else h.to(self.dtype)
+
+    def forward(self, stream: ResidualStream, step: StepContext, slot: LayerSlot) -> ResidualStream:
+        from ..ops.gated import residual_add
+
+        if stream.pending_norm is not None or stream.row_addend is not None:
+            raise RuntimeError("this block reads the sum itself: what is pending must be a plain addend")
+        if stream.pending is not None:
+            residual_add(stream.h, stream.pending)
+            stream.pending = None
+        h = stream.h
+        step.residual = None                 # a sublayer's result is normed before it joins the sum
+        mixer_slot = slot.by_part.get(self.names["mixer"], slot)
+        if self.filter is not None:
+            x = self.filter.forward(h, step, slot.by_part.get(self.names["filter"]))
+        else:
+            x = self._rounded(h)
+        y = self.mixer.forward(x, step, mixer_slot)
+        wants_copy = self.ffn is not None and self.dtype != torch.float32
+        x = self.norm1.add_normed(h, y, self.dtype if wants_copy else None)
+        if self.ffn is not None:
+            y = self.ffn.forward(x if wants_copy else h, step)
+            self.norm2.add_normed(h, y)
+        return stream
+
+
 register_part("block", "sandwich", SandwichBlock)
+register_part("block", "post_norm", PostNormBlock)
 register_part("block", "pre_norm", PreNormBlock)
 register_part("block", "parallel", ParallelBlock)

@@ -9,7 +9,7 @@ import torch
 from ..ops.linear import gate_up_swiglu, linear_into
 from .base import FeedForward, ParamSpec, StepContext, register_part
 
-__all__ = ["SwiGLU", "ClampedGatedFF"]
+__all__ = ["SwiGLU", "ClampedGatedFF", "PlainFF"]
 
 
 class SwiGLU(FeedForward):
@@ -114,5 +114,63 @@ class ClampedGatedFF(FeedForward):
         return linear_into(step.residual if step is not None else None, act, self.w_down)
 
 
+class PlainFF(FeedForward):
+    """``down(act(up(x)))`` without gate or biases.
+
+    params: ``hidden_size``, ``intermediate_size``, ``activation``: ``"relu2"`` (the square of relu) or
+    ``"normed_powers"`` (``a N(z) + b N(z^2) + c N(z^3) + e`` with powers taken element by element and ``N`` dividing
+    a token's row by its root mean square, ``eps`` inside the root; the four numbers are a tensor of the part),
+    ``eps`` (for the normed powers), ``names`` (local names of the up and down matrices and the activation's
+    tensor; default ``up_proj``, ``down_proj``, ``act``).
+    """
+
+    graph_safe = True
+
+    def __init__(self, params, dtype, device):
+        super().__init__(dtype, device)
+        self.hidden = int(params["hidden_size"])
+        self.inter = int(params["intermediate_size"])
+        self.activation = str(params["activation"])
+        if self.activation not in ("relu2", "normed_powers"):
+            raise ValueError(f"activation {self.activation!r}; known: relu2, normed_powers")
+        self.eps = float(params.get("eps", 0.0))
+        names = dict(params.get("names") or {})
+        self.names = {"up": names.get("up", "up_proj"), "down": names.get("down", "down_proj"), "act": names.get("act", "act")}
+        self.w_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+        self.coeff: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = {f"{self.names['up']}.weight": ParamSpec((self.inter, self.hidden)),
+                 f"{self.names['down']}.weight": ParamSpec((self.hidden, self.inter))}
+        if self.activation == "normed_powers":
+            specs[f"{self.names['act']}.weight"] = ParamSpec((4,), "vector", init="around_one")
+        return specs
+
+    def load(self, tensors):
+        self.w_up = tensors[f"{self.names['up']}.weight"]
+        self.w_down = tensors[f"{self.names['down']}.weight"]
+        self.coeff = tensors.get(f"{self.names['act']}.weight")
+
+    def named_weights(self) -> Dict[str, torch.Tensor]:
+        out = {f"{self.names['up']}.weight": self.w_up, f"{self.names['down']}.weight": self.w_down}
+        if self.coeff is not None:
+            out[f"{self.names['act']}.weight"] = self.coeff
+        return out
+
+    def forward(self, x, step: StepContext):
+        from ..ops import rownorm
+        from ..ops.linear import linear
+
+        z = linear(x, self.w_up)
+        z = z if z.is_contiguous() else z.contiguous()
+        if self.activation == "relu2":
+            act = rownorm.squared_relu_(z)
+        else:
+            act = rownorm.normed_powers(z, self.coeff, self.eps, self.dtype)
+        return linear_into(step.residual if step is not None else None, act, self.w_down)
+
+
 register_part("ffn", "swiglu", SwiGLU)
+register_part("ffn", "plain", PlainFF)
 register_part("ffn", "clamped_gated", ClampedGatedFF)

@@ -29,7 +29,9 @@ class RoutedExperts(FeedForward):
     ``alpha`` (default 1), ``limit`` (None: no clamps), ``shift`` (default 0), ``groups`` and ``keep``
     (default 1 and 1: no groups), ``scale`` (default 1), ``score`` (``"sigmoid"`` or ``"softmax"``),
     ``normalize`` (default True), ``floor`` (added to the sum the weights are divided by, default 1e-20),
-    ``shared`` (a :class:`PartSpec` of category ``ffn`` that every token runs through, or None), ``names``
+    ``shared`` (a :class:`PartSpec` of category ``ffn`` that every token runs through, or None),
+    ``expert_kind`` (``"gated"``, the default, or ``"plain"``: an expert is ``down(act(up(x)))`` with ``activation``
+    ``"relu2"``, the square of relu, and has no gate matrix), ``names``
     (``router``, ``expert`` with ``{}`` for the index, ``gate``, ``up``, ``down``, ``shared``; defaults
     ``router``, ``experts.{}``, ``gate_proj``, ``up_proj``, ``down_proj``, ``shared``).
 
@@ -56,6 +58,12 @@ class RoutedExperts(FeedForward):
         self.score = str(params.get("score", "sigmoid"))
         self.normalize = bool(params.get("normalize", True))
         self.floor = float(params.get("floor", 1e-20))
+        self.expert_kind = str(params.get("expert_kind", "gated"))
+        self.activation = params.get("activation")
+        if self.expert_kind not in ("gated", "plain"):
+            raise ValueError(f"expert kind {self.expert_kind!r}; known: gated, plain")
+        if self.expert_kind == "plain" and self.activation not in moe_ops.PLAIN_ACTS:
+            raise ValueError(f"a plain expert's activation {self.activation!r}; known: {sorted(map(str, moe_ops.PLAIN_ACTS))}")
         if self.score not in moe_ops.SCORE_FUNCTIONS:
             raise ValueError(f"router score {self.score!r}; known: {sorted(moe_ops.SCORE_FUNCTIONS)}")
         if self.groups <= 0 or self.experts % self.groups:
@@ -73,7 +81,7 @@ class RoutedExperts(FeedForward):
         shared: Optional[PartSpec] = params.get("shared")
         self.shared: Optional[Part] = None if shared is None else build_part("ffn", shared, dtype, device)
         self.w_router: Optional[torch.Tensor] = None
-        self.w_gate_up: Optional[torch.Tensor] = None   # [E, 2 ff, hidden]
+        self.w_gate_up: Optional[torch.Tensor] = None   # [E, 2 ff, hidden]; plain experts: [E, ff, hidden], up rows only
         self.w_down: Optional[torch.Tensor] = None      # [E, hidden, ff]
 
     def sub_parts(self) -> Dict[str, Part]:
@@ -85,23 +93,30 @@ class RoutedExperts(FeedForward):
     def param_specs(self) -> Dict[str, ParamSpec]:
         specs = {f"{self.names['router']}.weight": ParamSpec((self.experts, self.hidden))}
         for e in range(self.experts):
-            specs[self._expert(e, "gate")] = ParamSpec((self.inter, self.hidden))
+            if self.expert_kind == "gated":
+                specs[self._expert(e, "gate")] = ParamSpec((self.inter, self.hidden))
             specs[self._expert(e, "up")] = ParamSpec((self.inter, self.hidden))
             specs[self._expert(e, "down")] = ParamSpec((self.hidden, self.inter))
         return specs
 
     def load(self, tensors):
         self.w_router = tensors[f"{self.names['router']}.weight"]
-        both = [torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], dim=0)
-                for e in range(self.experts)]
+        if self.expert_kind == "gated":
+            both = [torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], dim=0)
+                    for e in range(self.experts)]
+        else:
+            both = [tensors[self._expert(e, "up")] for e in range(self.experts)]
         self.w_gate_up = torch.stack(both).contiguous()
         self.w_down = torch.stack([tensors[self._expert(e, "down")] for e in range(self.experts)]).contiguous()
 
     def named_weights(self) -> Dict[str, torch.Tensor]:
         out = {f"{self.names['router']}.weight": self.w_router}
         for e in range(self.experts):
-            out[self._expert(e, "gate")] = self.w_gate_up[e, :self.inter]
-            out[self._expert(e, "up")] = self.w_gate_up[e, self.inter:]
+            if self.expert_kind == "gated":
+                out[self._expert(e, "gate")] = self.w_gate_up[e, :self.inter]
+                out[self._expert(e, "up")] = self.w_gate_up[e, self.inter:]
+            else:
+                out[self._expert(e, "up")] = self.w_gate_up[e]
             out[self._expert(e, "down")] = self.w_down[e]
         return out
 
@@ -116,8 +131,11 @@ class RoutedExperts(FeedForward):
         ids, weights = self.route(x)
         order, offsets = moe_ops.sort_pairs(ids, self.experts)
         pairs = n * self.top
-        act = moe_ops.expert_products(x, self.w_gate_up, order, offsets, pairs, self.top, self.dtype,
-                                      gated=(self.alpha, self.limit, self.shift))
+        if self.expert_kind == "gated":
+            how = dict(gated=(self.alpha, self.limit, self.shift))
+        else:
+            how = dict(act=self.activation)
+        act = moe_ops.expert_products(x, self.w_gate_up, order, offsets, pairs, self.top, self.dtype, **how)
         # few pairs: the float32 sums as they are; many: one rounding, half the traffic
         y = moe_ops.expert_products(act, self.w_down, order, offsets, pairs, 1,
                                     torch.float32 if pairs <= FLOAT32_PAIRS else self.dtype)

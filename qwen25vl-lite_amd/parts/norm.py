@@ -10,7 +10,7 @@ from ..ops import kernels, skinny
 from ..ops.linear import NormedRows
 from .base import Norm, ParamSpec, ResidualStream, register_part
 
-__all__ = ["RMSNorm"]
+__all__ = ["RMSNorm", "LayerNorm"]
 
 
 class RMSNorm(Norm):
@@ -58,4 +58,44 @@ class RMSNorm(Norm):
         return out
 
 
+class LayerNorm(Norm):
+    """``(x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * weight``: the mean is taken off, there is no
+    bias; statistics in float32, the deviations formed from the mean (two passes).
+
+    params: ``size`` (row width), ``eps``.
+    """
+
+    graph_safe = True
+
+    def __init__(self, params, dtype, device):
+        super().__init__(dtype, device)
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.size,), "vector", init="around_one")}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"]
+
+    def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None, lazy: bool = False):
+        from ..ops import rownorm
+        from ..ops.gated import residual_add
+
+        if stream.pending_norm is not None or stream.row_addend is not None:
+            raise RuntimeError("a layer norm does not fold a normed addend or a pass vector into the sum")
+        if stream.pending is not None:
+            residual_add(stream.h, stream.pending)
+            stream.pending = None
+        return rownorm.layer_norm(stream.h, self.weight, self.eps, self.dtype, rows=rows)
+
+    def add_normed(self, h: torch.Tensor, y: torch.Tensor, copy_dtype: Optional[torch.dtype] = None):
+        """``h += norm(y)`` in float32, in place; with ``copy_dtype`` the new ``h`` is also returned in it."""
+        from ..ops import rownorm
+
+        return rownorm.layer_norm_add_(h, y, self.weight, self.eps, copy_dtype)
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "layer_norm", LayerNorm)

@@ -9,9 +9,9 @@ import torch
 
 from ..ops import kernels
 from ..ops.linear import linear
-from .base import Embedding, Head, ParamSpec, register_part
+from .base import Embedding, Head, ParamSpec, Part, PartSpec, build_part, register_part
 
-__all__ = ["TokenTable", "LinearHead"]
+__all__ = ["TokenTable", "NormedTokenTable", "LinearHead"]
 
 
 class TokenTable(Embedding):
@@ -35,6 +35,31 @@ class TokenTable(Embedding):
 
     def forward(self, token_ids, step):
         return kernels.embed_gather(token_ids, self.table)
+
+
+class NormedTokenTable(TokenTable):
+    """A token's row of the table, normed: the residual sum starts at ``norm(table[id])`` in float32.
+
+    params: ``vocab_size``, ``hidden_size``, ``norm`` (a :class:`PartSpec` of a norm that has a ``weight`` and an
+    ``eps``: a layer norm), ``norm_name`` (the norm's checkpoint sub-name, default ``norm``).
+    """
+
+    def __init__(self, params, dtype, device):
+        super().__init__(params, dtype, device)
+        spec: PartSpec = params["norm"]
+        if spec.kind != "layer_norm":
+            raise ValueError("the norm on the token table is a layer norm")
+        self.norm = build_part("norm", spec, dtype, device)
+        self.norm_name = str(params.get("norm_name", "norm"))
+
+    def sub_parts(self) -> Dict[str, Part]:
+        return {self.norm_name: self.norm}
+
+    def forward(self, token_ids, step):
+        from ..ops import rownorm
+
+        rows = kernels.embed_gather(token_ids, self.table)
+        return rownorm.layer_norm(rows, self.norm.weight, self.norm.eps, torch.float32)
 
 
 class LinearHead(Head):
@@ -73,4 +98,5 @@ class LinearHead(Head):
 
 
 register_part("embedding", "token_table", TokenTable)
+register_part("embedding", "normed_table", NormedTokenTable)
 register_part("head", "linear", LinearHead)

@@ -30,6 +30,10 @@ def _seed_for(seed: int, name: str) -> int:
 def _draw(name: str, shape, seed: int, std: float, device, dtype: torch.dtype, init: str = "normal") -> torch.Tensor:
     if init in ("zeros", "ones"):
         return torch.full(tuple(shape), float(init == "ones"), dtype=dtype, device=device)
+    if init == "unit_interval":
+        gen = torch.Generator(device=device)
+        gen.manual_seed(_seed_for(seed, name))
+        return torch.empty(tuple(shape), dtype=torch.float32, device=device).uniform_(0.0, 1.0, generator=gen).to(dtype)
     if init not in ("normal", "around_one"):
         raise ValueError(f"{name}: no rule to draw a tensor with init {init!r}")
     gen = torch.Generator(device=device)
