@@ -220,6 +220,7 @@ __global__ __launch_bounds__(256) void attn_window_kernel(WindowArgs a) {
 #pragma unroll
         for (int dt = 0; dt < NT; ++dt) acc[c][dt] += *reinterpret_cast<const f32x4_t*>(s_acc[w][c * NT + dt][lane]) * f;
       }
+      m[c] = m_safe;                                       // what the sums now refer to
     }
   }
 #pragma unroll

@@ -45,6 +45,13 @@ LIBRARIES = [
     ("attention_window", {"HD": 16, "VD": 16}),
     ("attention_window", {"HD": 64, "VD": 32}),
     ("attention_window", {"HD": 8, "VD": 8}),
+    # one key/value head whose values are the first channels of its keys (attention through a latent)
+    ("attention_window", {"HD": 32, "VD": 24}),
+    ("attention_window", {"HD": 56, "VD": 40}),
+    ("attention_window", {"HD": 32, "VD": 16}),
+    ("attention_window", {"HD": 24, "VD": 16}),
+    ("attention_window", {"HD": 128, "VD": 64}),
+    ("attention_window", {"HD": 40, "VD": 24}),
     # the kind whose waves carry three column tiles (long prompts)
     ("attention_mfma", {"HD": 128, "BLK_CT": 3}),
     ("attention_mfma", {"HD": 48, "BLK_CT": 3}),

@@ -47,13 +47,13 @@ def _rel(got, want):
     return _rel_rows(got, want).max().item()
 
 
-def _like_rounding(errors, rounding):
+def _like_rounding(errors, rounding, slack=1e-3):
     """``errors``: per-row distances of the engine's bfloat16 logits from exact arithmetic; ``rounding``:
     the same for the plain model with its stored activations rounded to bfloat16.  Rounding moves single
     rows far (a router's choice between two experts whose scores all but tie falls the other way), in the
     plain model as in the engine, so the two are compared as distributions."""
-    return (errors.median() < 2 * rounding.median() + 1e-3
-            and errors.quantile(0.9) < 3 * rounding.quantile(0.9) + 1e-3)
+    return (errors.median() < 2 * rounding.median() + slack
+            and errors.quantile(0.9) < 3 * rounding.quantile(0.9) + slack)
 
 
 def _replayer(folder, dtype, max_tokens, max_live=4):
@@ -229,26 +229,35 @@ def test_hgrn2_alone_whole_in_steps_and_in_chunks(heads, dim, vdim, dtype, tmp_p
 
 
 def test_a_slow_channel_remembers_a_far_token(tmp_path):
-    """One key channel of the recurrence is made to forget almost nothing (a floor of 0.999) and is the only one
+    """One key channel of the recurrence is made to forget almost nothing (a floor of 0.98) and is the only one
     the late queries read: what token 3 wrote is still there 250 tokens on, and a state lost on the way
     (a slot cleared, a chunk's carry dropped) would show."""
     heads, dim, vdim = 2, 8, 8
 
     def edit(t):
         low = torch.full((heads * dim,), 0.05)
-        low[0] = 0.999
+        low[::dim] = 0.98                       # the first channel of every head
         t["l0.mix.lower"] = low.to(torch.bfloat16)
+        gate, bias = t["l0.mix.f"].clone(), t["l0.mix.f.b"].clone()
+        gate[::dim] = 0                         # its gate stands at the floor plus half the rest, whatever the token
+        bias[::dim] = 0
+        t["l0.mix.f"], t["l0.mix.f.b"] = gate, bias
+        q = t["l0.mix.q"].clone()
+        keep = torch.zeros(heads * dim, 1, dtype=q.dtype)
+        keep[::dim] = 1
+        t["l0.mix.q"] = q * keep                # queries read that channel only
     runner, blocks, t = _one_layer(tmp_path, ru.layer(ru.hgrn2(heads, dim, vdim)), tensors_edit=edit)
     mixer = blocks[0].mixer
     torch.manual_seed(9)
     n = 260
     x = torch.randn(n, 56, dtype=F64)
+    x[3] *= 30.0                                # a token that writes much
     m = ru.hgrn2(heads, dim, vdim)["mixer"]
     want = plain.hgrn2(x, t, "l0.mix.", m, 1e-4)
     x2 = x.clone()
     x2[3] = -x[3]
     moved = plain.hgrn2(x2, t, "l0.mix.", m, 1e-4)
-    assert (moved[-5:] - want[-5:]).abs().max() > 1e-3 * want.abs().max()    # the far token matters to the end
+    assert (moved[-5:] - want[-5:]).abs().max() > 1e-2 * want.abs().max()    # the far token matters to the end
     pieces, at = [], 0
     for size in (5, 140, 1, 1, 100, 13):
         step = _step_for(runner, [("s", size, at)])
@@ -361,8 +370,8 @@ def test_squared_relu_experts_alone(dtype, width, ff, rows, tmp_path):
     x = torch.randn(rows, width, dtype=F64)
     store = plain._keep if dtype == torch.float32 else plain.to_bfloat16_and_back
     want = plain.moe_ff(store(x), t, "l0.mlp.", mlp, store)
-    step = _step_for(runner, [("a", rows, 0)]) if rows <= 512 else None
-    got = blocks[0].ffn.forward(x.to(dtype).cuda(), step)
+    from types import SimpleNamespace
+    got = blocks[0].ffn.forward(x.to(dtype).cuda(), SimpleNamespace(residual=None))
     got = (got.sum(0) if got.dim() == 3 else got).double().cpu()
     if dtype == torch.float32:
         assert torch.allclose(got, want, atol=2e-5 * want.abs().max().item())
@@ -388,7 +397,7 @@ def test_dense_feed_forward_alone(dtype, tmp_path):
 # ---------------------------------------------------------------------------------------------
 # the attention kernels with a sink, against dense masked attention
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("hd, vd, nq, ps", [(32, 24, 3, 16), (128, 96, 6, 16), (64, 32, 20, 16), (40, 24, 5, 16)])
+@pytest.mark.parametrize("hd, vd, nq, ps", [(32, 24, 3, 16), (128, 64, 7, 16), (64, 32, 20, 16), (40, 24, 5, 16)])
 @pytest.mark.parametrize("window", [9, 37, 70, None])
 def test_attention_with_a_sink_on_the_matrix_cores(hd, vd, nq, ps, window):
     """One key/value head whose values are the first channels of its keys, as the latent attention keeps them:
@@ -501,15 +510,18 @@ def test_peaked_attention_at_window_edges_and_far_keys(dtype, folders):
     folder = folders["sharp"]
     toks = random_tokens(330, ru.SHARP["vocab"], 40)
     want = _oracle(folder, toks)
-    rounding = _rel_rows(_oracle(folder, toks, plain.to_bfloat16_and_back), want)
+    if dtype == "float32":
+        # scores this large make float32 arithmetic itself visible: the measure is the plain model run in float32
+        cfg, t32 = plain.rapisun_read(folder, torch.float32)
+        rounding, slack = _rel_rows(plain.rapisun_forward(cfg, t32, toks), want), 1e-5
+    else:
+        rounding, slack = _rel_rows(_oracle(folder, toks, plain.to_bfloat16_and_back), want), 1e-3
     for steps in (tail_trace({"s": toks}, 70), portion_trace({"s": toks}, (64, 3, 41, 2, 17, 90))):
         got = _rows(run_steps(_replayer(folder, dtype, round64(len(toks))), steps), "s", len(toks))
-        if dtype == "float32":
-            assert _rel(got, want) < 2e-5
-        else:
-            errors = _rel_rows(got, want)
-            assert _like_rounding(errors, rounding), (errors.median(), rounding.median(), errors.quantile(0.9),
-                                                      rounding.quantile(0.9))
+        errors = _rel_rows(got, want)
+        assert _like_rounding(errors, rounding, slack), (errors.median(), rounding.median(), errors.quantile(0.9),
+                                                         rounding.quantile(0.9))
+        assert errors.max() < 4 * rounding.max() + slack, (errors.max(), rounding.max())
 
 
 def test_sharpening_matters(folders):
