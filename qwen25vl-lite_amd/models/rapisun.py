@@ -100,7 +100,7 @@ class RapisunConfig:
                 dims, rot_dim = int(m["rot"]["dims"]), int(m["rot_dim"])
                 if rot_dim < 0 or dims < 0 or dims % 2 or dims > rot_dim:
                     raise ConfigError(f"config.json: {where}.mixer.rot.dims must be even and at most rot_dim")
-                if m.get("mask"):
+                if m.get("mask") is not None:
                     _need(m["mask"], ("size",), f"{where}.mixer.mask")
                     _positive(m["mask"], ("size",), f"{where}.mixer.mask")
                 src = m.get("kv_from")
@@ -154,7 +154,7 @@ def _map_name(name: str) -> str:
 
 
 def _window(m: Dict[str, Any]) -> Optional[int]:
-    return int(m["mask"]["size"]) if m.get("mask") else None
+    return int(m["mask"]["size"]) if m.get("mask") is not None else None
 
 
 def retained_keys(layers: List[Dict[str, Any]]) -> Dict[int, Optional[int]]:
