@@ -95,6 +95,42 @@ def dazapel_config(layers, size="7b", experts=32, top=6, window=1024, keep_first
             "residual_mult": 0.5, "layers": [{"type": "attention", "mixer": mixer(i), "mlp": mlp} for i in range(int(layers))]}
 
 
+RAPISUN_ORDER = ("hgrn2", "latent", "latent_shared", "hgrn2")
+
+
+def rapisun_config(layers, size="7b", order=RAPISUN_ORDER, experts=32, top=6, window=1024, kv_rank=192, rot_dim=64):
+    """A Rapisun decoder with the width, head count and vocabulary of one of SIZES.  Layers in the given order
+    (repeated): ``hgrn2`` (keys of 64, values of 128 channels a head), ``latent`` (attention through latents of
+    a quarter of the width for queries and ``kv_rank`` for keys and values, heads of 128 unrotated and
+    ``rot_dim`` rotated channels, the last ``window`` keys), ``latent_shared`` (the same, reading the cache of the
+    nearest ``latent`` layer before it).  The first layer of every round has the size's dense feed-forward, the
+    others routed experts of an eighth of its width, of which a token uses ``top``, and a shared expert twice as
+    wide: with 6 chosen a token runs through as many feed-forward channels as in the dense layer."""
+    s = SIZES[size]
+    nh, hd, width = s["num_attention_heads"], 128, s["hidden_size"]
+    ff = s["intermediate_size"] // 8 // 16 * 16
+    moe = {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": 2 * ff}, "router": {"experts": experts, "top": top}}
+    dense = {"kind": "dense", "ff": s["intermediate_size"]}
+    out, owner = [], None
+    for i in range(int(layers)):
+        kind = order[i % len(order)]
+        if kind == "hgrn2":
+            lay = {"type": "hgrn2", "mixer": {"heads": nh, "dim": hd // 2, "vdim": hd}}
+        else:
+            m = {"heads": nh, "dim": hd, "rot_dim": rot_dim, "vdim": hd, "q_rank": width // 4 // 16 * 16,
+                 "kv_rank": kv_rank, "scale": (hd + rot_dim) ** -0.5, "rot": {"base": 250000.0, "dims": rot_dim},
+                 "mask": {"size": window}}
+            if kind == "latent_shared" and owner is not None:
+                m["kv_from"] = owner
+            else:
+                owner = i
+            lay = {"type": "latent_attention", "mixer": m}
+        lay["mlp"] = dense if i % len(order) == 0 else moe
+        out.append(lay)
+    return {"architecture": "Rapisun", "width": width, "vocab": s["vocab_size"], "norm": {"eps": 1e-6},
+            "canon": {"taps": 4}, "layers": out}
+
+
 def step_bytes(t, batch, ctx, bytes_per_value=2):
     """Bytes a decode step has to read: every weight it uses once (all layers and the head; of the
     embedding only the rows looked up) and the keys and values of the live requests."""
@@ -249,11 +285,14 @@ def main(argv=None) -> int:
     ap.add_argument("--attention", type=int, nargs="+", metavar="TOKENS",
                     help="instead: the prefill attention alone (one request of that many tokens in one step, the "
                          "chosen size's heads, bfloat16, pages in shuffled order), microseconds and TFLOP/s for each length")
-    ap.add_argument("--design", choices=["gogudra", "dazapel"],
+    ap.add_argument("--design", choices=["gogudra", "dazapel", "rapisun"],
                     help="instead: prefill (2,048 tokens) and decode throughput of this design at the chosen size's "
                          "width, heads and feed-forward (random weights), beside the Qwen2.5-VL decoder with as many layers")
-    ap.add_argument("--order", default="gla,gla,lightning,attention",
-                    help="with --design: the mixers of successive layers, repeated")
+    ap.add_argument("--beside", choices=["qwen25vl", "gogudra", "dazapel"], default="qwen25vl",
+                    help="with --design: the model the design is measured beside, at the same sizes")
+    ap.add_argument("--order", default=None,
+                    help="with --design gogudra or rapisun: the mixers of successive layers, repeated (gogudra: "
+                         "gla,gla,lightning,attention; rapisun: " + ",".join(RAPISUN_ORDER) + ")")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-lookahead", action="store_true",
                     help="do not queue the next decode step before the running one's tokens are known")
@@ -279,6 +318,8 @@ def main(argv=None) -> int:
 
     if args.design and not args.layers:
         args.layers = 8
+    if args.order is None:
+        args.order = ",".join(RAPISUN_ORDER) if args.design == "rapisun" else "gla,gla,lightning,attention"
     cfg = Qwen25VLConfig.from_dict(decoder_config(args.layers, args.size))
     t = cfg.text_config
     vocab = t.vocab_size
@@ -350,17 +391,24 @@ def main(argv=None) -> int:
 
     if args.design:
         from qwen25vl_lite_amd.config import load_config
-        out = {"metric": f"prefill and decode tok/s, {args.design} beside the Qwen2.5-VL decoder "
+        beside = "the Qwen2.5-VL decoder" if args.beside == "qwen25vl" else args.beside
+        out = {"metric": f"prefill and decode tok/s, {args.design} beside {beside} "
                          f"({args.size} sizes, {args.layers} layers, {args.dtype})", "unit": "tokens/s",
-               "order": args.order.split(",") if args.design == "gogudra" else None, "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
+               "order": args.order.split(",") if args.design in ("gogudra", "rapisun") else None, "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
         steps, warmup = min(args.steps, 64), min(args.warmup, 4)
-        for name in ("qwen25vl", args.design):
+        def design_config(name):
+            if name == "dazapel":
+                return dazapel_config(args.layers, args.size)
+            if name == "rapisun":
+                return rapisun_config(args.layers, args.size, tuple(args.order.split(",")))
+            return gogudra_config(args.layers, args.size, tuple(args.order.split(",")) if name == args.design
+                                  else ("gla", "gla", "lightning", "attention"))
+
+        for name in (args.beside, args.design):
             if name != "qwen25vl":
                 del model
                 torch.cuda.empty_cache()
-                design = (dazapel_config(args.layers, args.size) if args.design == "dazapel"
-                          else gogudra_config(args.layers, args.size, tuple(args.order.split(","))))
-                model = build_model(load_config(design), dtype, "cuda:0")
+                model = build_model(load_config(design_config(name)), dtype, "cuda:0")
                 fill_random(model, seed=0)
                 torch.cuda.synchronize()
             sec = prefill_rate(2048)

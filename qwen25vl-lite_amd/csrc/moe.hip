@@ -175,7 +175,8 @@ struct ExpertArgs {
   const void* w;        // [E, rows_w, K]
   const int* sorted;
   const int* offsets;
-  void* out;            // [P, R]
+  void* out;            // [P, R], rows ldo values apart
+  long long ldo;
   int P, E, R, K, div, gated;
   int act;              // on a plain product's values: 0 none, 1 the square of relu
   float alpha, limit, shift;
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(256) void moe_rows_kernel(ExpertArgs a) {
     } else {
       g = plain_value(g, a.act);
     }
-    if (lane == 0) stf<TO>((TO*)a.out + (size_t)p * a.R + c, g);
+    if (lane == 0) stf<TO>((TO*)a.out + (size_t)p * a.ldo + c, g);
   }
 }
 
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(256) void moe_mfma_kernel(ExpertArgs a) {
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     if (pair[t] < 0) continue;
-    TO* o = (TO*)a.out + (size_t)pair[t] * a.R + c0 + 4 * lg;
+    TO* o = (TO*)a.out + (size_t)pair[t] * a.ldo + c0 + 4 * lg;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (c0 + 4 * lg + j >= a.R) break;
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(ExpertArgs a, int tiles_m
     const int i = first + wm * 64 + m * 16 + r;
     if (i >= last) continue;
     const int pair = a.sorted[i];
-    TO* o = (TO*)a.out + (size_t)pair * a.R;
+    TO* o = (TO*)a.out + (size_t)pair * a.ldo;
 #pragma unroll
     for (int n = 0; n < (GATED ? NW / 2 : NW); ++n) {
       const int c = c0 + wn * PER_WAVE + n * 16 + 4 * lg;
@@ -611,7 +612,7 @@ __global__ __launch_bounds__(256) void moe_stream_kernel(ExpertArgs a, int tiles
     const int i = first + wm * 64 + m * 16 + r;
     if (i >= last) continue;
     const int pair = a.sorted[i];
-    TO* o = (TO*)a.out + (size_t)pair * a.R;
+    TO* o = (TO*)a.out + (size_t)pair * a.ldo;
 #pragma unroll
     for (int n = 0; n < (GATED ? ST_NW / 2 : ST_NW); ++n) {
       const int c = c0 + wn * PER_WAVE + n * 16 + 4 * lg;
@@ -631,13 +632,14 @@ __global__ __launch_bounds__(256) void moe_stream_kernel(ExpertArgs a, int tiles
 // write either.  The matrix-core kernel runs for bfloat16 with K a multiple of 8 and rows of x on
 // 16-byte boundaries; `big_tiles` asks for the kernel with tiles of 128 pairs through LDS (many pairs an expert).
 extern "C" int qvl_moe_experts(const void* x, long long ldx, int x_dtype, const void* w, const void* sorted,
-                               const void* offsets, void* out, int out_dtype, int P, int E, int R, int K, int div,
+                               const void* offsets, void* out, long long ldo, int out_dtype, int P, int E, int R, int K,
+                               int div,
                                int gated, float alpha, float limit, float shift, int act, int big_tiles,
                                hipStream_t stream) {
   if (P <= 0) return QVL_OK;
-  if (E <= 0 || R <= 0 || K <= 0 || div <= 0 || ldx < K || !x || !w || !sorted || !offsets || !out) return QVL_ERR_SHAPE;
+  if (E <= 0 || R <= 0 || K <= 0 || div <= 0 || ldx < K || ldo < R || !x || !w || !sorted || !offsets || !out) return QVL_ERR_SHAPE;
   ExpertArgs a;
-  a.x = x; a.ldx = ldx; a.w = w; a.sorted = (const int*)sorted; a.offsets = (const int*)offsets; a.out = out;
+  a.x = x; a.ldx = ldx; a.w = w; a.sorted = (const int*)sorted; a.offsets = (const int*)offsets; a.out = out; a.ldo = ldo;
   a.P = P; a.E = E; a.R = R; a.K = K; a.div = div; a.gated = gated; a.act = gated ? 0 : act; a.alpha = alpha; a.limit = limit; a.shift = shift;
   if (x_dtype == 1 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0) {
     if (out_dtype != 0 && out_dtype != 1) return QVL_ERR_DTYPE;

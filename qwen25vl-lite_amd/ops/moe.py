@@ -15,7 +15,7 @@ import torch
 
 from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
 
-__all__ = ["route", "sort_pairs", "expert_products", "combine", "SCORE_FUNCTIONS", "BIG_TILE_PAIRS"]
+__all__ = ["route", "sort_pairs", "pairs_by_column", "expert_products", "combine", "SCORE_FUNCTIONS", "BIG_TILE_PAIRS"]
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 SCORE_FUNCTIONS = {"sigmoid": 0, "softmax": 1}
@@ -61,15 +61,25 @@ def sort_pairs(ids: torch.Tensor, num_experts: int) -> Tuple[torch.Tensor, torch
     return order, offsets
 
 
+def pairs_by_column(rows: int, columns: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(order, offsets)`` as :func:`sort_pairs` gives them for ``ids[row, c] = c``: pair ``row * columns + c``
+    belongs to "expert" ``c``.  With it :func:`expert_products` multiplies slice ``c`` of every row of a
+    ``[rows, columns, K]`` tensor by a matrix of its own (a product per head)."""
+    order = torch.arange(rows * columns, dtype=torch.int32, device=device).view(rows, columns).t().contiguous().view(-1)
+    offsets = torch.arange(columns + 1, dtype=torch.int32, device=device) * rows
+    return order, offsets
+
+
 def expert_products(x: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, offsets: torch.Tensor, pairs: int,
                     div: int, out_dtype: torch.dtype, gated: Optional[Tuple[float, Optional[float], float]] = None,
-                    act: Optional[str] = None) -> torch.Tensor:
+                    act: Optional[str] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[p] = x[p // div] @ weight[e(p)].T`` for every pair ``p``, ``e(p)`` the expert whose range
     of ``order`` holds it; ``weight`` is ``[E, R, K]``.  With ``gated = (alpha, limit, shift)``,
     ``weight`` is ``[E, 2 R, K]`` (R gate rows, then R up rows) and
     ``out[p] = g sigmoid(alpha g) (u + shift)`` with ``g`` capped at ``limit`` and ``u`` clamped to
     ``[-limit, limit]`` (``limit`` None: no clamps).  Without ``gated``, ``act`` ``"relu2"`` squares the positive
-    part of every value of the product.  Returns ``[pairs, R]`` in ``out_dtype``."""
+    part of every value of the product.  Returns ``[pairs, R]`` in ``out_dtype``; with ``out`` (``[pairs, R]`` of
+    that dtype, rows any number of values apart) the result goes there."""
     _dev(x, weight, order, offsets)
     _need(weight.dim() == 3 and weight.is_contiguous() and x.dim() == 2 and x.stride(1) == 1
           and x.dtype == weight.dtype and x.shape[1] == weight.shape[2], "x [M, K] and weight [E, rows, K] of one dtype")
@@ -82,13 +92,17 @@ def expert_products(x: torch.Tensor, weight: torch.Tensor, order: torch.Tensor, 
     _need(pairs <= x.shape[0] * div, "a pair's row lies outside x")
     _need(out_dtype == x.dtype or (x.dtype == torch.bfloat16 and out_dtype == torch.float32),
           "float32 operands give float32; bfloat16 operands give either")
-    out = torch.empty((pairs, r), dtype=out_dtype, device=x.device)
+    if out is None:
+        out = torch.empty((pairs, r), dtype=out_dtype, device=x.device)
+    _dev(out)
+    _need(out.dtype == out_dtype and tuple(out.shape) == (pairs, r) and out.stride(1) == 1 and out.stride(0) >= r,
+          "out must be [pairs, R] of the output's dtype with contiguous rows")
     alpha, limit, shift = gated if gated else (1.0, None, 0.0)
-    fn = _fn("moe", "qvl_moe_experts", [_c_ptr, _c_ll, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-                                        _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _c_int,
+    fn = _fn("moe", "qvl_moe_experts", [_c_ptr, _c_ll, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int,
+                                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _c_int,
                                         _c_ptr])
     _check(fn(_ptr(x), x.stride(0), dtype_code(x.dtype), _ptr(weight), _ptr(order), _ptr(offsets), _ptr(out),
-              dtype_code(out_dtype), int(pairs), e, r, k, int(div), int(bool(gated)), float(alpha), float(limit or 0.0),
+              out.stride(0), dtype_code(out_dtype), int(pairs), e, r, k, int(div), int(bool(gated)), float(alpha), float(limit or 0.0),
               float(shift), PLAIN_ACTS[act], int(pairs >= BIG_TILE_PAIRS * e), _stream()), "moe experts")
     return out
 

@@ -7,7 +7,9 @@ With ``c`` the normed key/value latent and ``r`` the rotated key part of a key, 
 (Uk_h^T q_plain) . c``, the query is carried into the latent's space once per token and head, and attention
 runs over one cached key ``[c | r]`` per token, shared by all heads, whose value is ``c`` itself; the
 value up-projection ``Uv_h`` is applied to the attended latent.  The pages, block tables and attention
-kernels are the engine's own (one key/value head, values narrower than keys).
+kernels are the engine's own (one key/value head, values narrower than keys).  The two products with a
+matrix per head run through the kernels of the routed experts, a head taking an expert's place: they read
+and write a head's slice of a token's row where it lies, so nothing is transposed or copied.
 """
 
 from __future__ import annotations
@@ -16,7 +18,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..ops import kernels, latent
+from ..ops import kernels, latent, moe as moe_ops
 from ..ops.attention import paged_attention
 from ..ops.linear import linear, linear_into
 from .base import CacheNeed, LayerSlot, Mixer, ParamSpec, PartSpec, StepContext, build_part, register_part
@@ -71,7 +73,7 @@ class LatentAttention(Mixer):
         self.q_norm: Optional[torch.Tensor] = None
         self.kv_norm: Optional[torch.Tensor] = None
         self.w_uq: Optional[torch.Tensor] = None        # [heads (dim + rot_dim), q_rank]
-        self.w_uk: Optional[torch.Tensor] = None        # [heads, dim, kv_rank]
+        self.w_uk_t: Optional[torch.Tensor] = None      # [heads, kv_rank, dim]: Uk_h^T, the matrix that carries a query over
         self.w_uv: Optional[torch.Tensor] = None        # [heads, vdim, kv_rank]
         self.sink: Optional[torch.Tensor] = None
         self.w_out: Optional[torch.Tensor] = None
@@ -107,7 +109,7 @@ class LatentAttention(Mixer):
         self.w_down = torch.cat(mats, dim=0).contiguous()
         self.q_norm = tensors[f"{n['dq_norm']}.weight"]
         self.w_uq = tensors[f"{n['uq']}.weight"]
-        self.w_uk = tensors[f"{n['uk']}.weight"].view(self.heads, self.dim, self.kv_rank)
+        self.w_uk_t = tensors[f"{n['uk']}.weight"].view(self.heads, self.dim, self.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = tensors[f"{n['uv']}.weight"].view(self.heads, self.vdim, self.kv_rank)
         self.sink = tensors.get(f"{n['sink']}.weight")
         self.w_out = tensors[f"{n['o']}.weight"]
@@ -115,7 +117,7 @@ class LatentAttention(Mixer):
     def named_weights(self) -> Dict[str, torch.Tensor]:
         n = self.names
         out = {f"{n['dq']}.weight": self.w_down[:self.q_rank], f"{n['dq_norm']}.weight": self.q_norm,
-               f"{n['uq']}.weight": self.w_uq, f"{n['uk']}.weight": self.w_uk.reshape(-1, self.kv_rank),
+               f"{n['uq']}.weight": self.w_uq, f"{n['uk']}.weight": self.w_uk_t.transpose(1, 2).reshape(-1, self.kv_rank),
                f"{n['uv']}.weight": self.w_uv.reshape(-1, self.kv_rank), f"{n['o']}.weight": self.w_out}
         if not self.kv_shared:
             out[f"{n['dkv']}.weight"] = self.w_down[self.q_rank:]
@@ -156,13 +158,15 @@ class LatentAttention(Mixer):
         q = q if q.is_contiguous() else q.contiguous()
         # the query in the latent's space, head by head: [N, heads, kv_rank | rot_dim]
         q_lat = torch.empty((n, h, r + rot), dtype=self.dtype, device=x.device)
-        torch.bmm(q.view(n, h, self.dim + rot)[:, :, :self.dim].transpose(0, 1), self.w_uk,
-                  out=q_lat[:, :, :r].transpose(0, 1))
+        by_head = step.per_pass.get(("pairs_by_head", h))
+        if by_head is None:
+            by_head = step.per_pass[("pairs_by_head", h)] = moe_ops.pairs_by_column(n, h, x.device)
+        moe_ops.expert_products(q.view(n * h, self.dim + rot)[:, :self.dim], self.w_uk_t, *by_head, n * h, 1, self.dtype,
+                                out=q_lat.view(n * h, r + rot)[:, :r])
         latent.latent_query_rotate_(q, h, self.dim, rot, r, cs, q_lat)
         o_lat = paged_attention(q_lat.view(n, h * (r + rot)), slot.k_cache, slot.v_cache, group.block_table, step, h,
                                 self.window, self.scale, sinks=self.sink)
-        o = torch.empty((n, h, self.vdim), dtype=self.dtype, device=x.device)
-        torch.bmm(o_lat.view(n, h, r).transpose(0, 1), self.w_uv.transpose(1, 2), out=o.transpose(0, 1))
+        o = moe_ops.expert_products(o_lat.view(n * h, r), self.w_uv, *by_head, n * h, 1, self.dtype)
         return linear_into(step.residual, o.view(n, h * self.vdim), self.w_out)
 
 

@@ -357,6 +357,29 @@ def test_softmax_router(e, top):
     assert torch.allclose(wts.cpu().double().gather(1, order), w.gather(1, idx.argsort(dim=-1)), atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype, heads, k, r", [(torch.float32, 3, 12, 20), (torch.bfloat16, 5, 24, 40), (torch.bfloat16, 28, 128, 192),
+                                               (torch.bfloat16, 2, 64, 96), (torch.bfloat16, 3, 20, 7)])
+@pytest.mark.parametrize("rows", [1, 9, 70, 300])
+def test_a_product_per_head_on_slices_of_rows(dtype, heads, k, r, rows):
+    """``out[n, h, :r] = x[n, h, :k] @ w[h].T`` where a head's slice is part of a longer row, on both sides:
+    what lies beside the slices stays as it was."""
+    from qwen25vl_lite_amd.ops import moe as moe_ops
+    torch.manual_seed(rows + heads)
+    x = torch.randn(rows, heads, k + 8).to(dtype).cuda()
+    w = (torch.randn(heads, r, k) / k ** 0.5).to(dtype).cuda()
+    out = torch.full((rows, heads, r + 16), 7.0, dtype=dtype, device="cuda")
+    order, offsets = moe_ops.pairs_by_column(rows, heads, "cuda")
+    moe_ops.expert_products(x.view(rows * heads, k + 8)[:, :k], w, order, offsets, rows * heads, 1, dtype,
+                            out=out.view(rows * heads, r + 16)[:, :r])
+    want = torch.einsum("nhk,hrk->nhr", x[:, :, :k].double(), w.double())
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert (out[:, :, :r].double() - want).abs().max() < tol * max(1.0, want.abs().max().item())
+    assert torch.all(out[:, :, r:] == 7.0)
+    # and into a tensor of its own
+    y = moe_ops.expert_products(x.view(rows * heads, k + 8)[:, :k], w, order, offsets, rows * heads, 1, dtype)
+    assert y.is_contiguous() and torch.equal(y.view(rows, heads, r), out[:, :, :r])
+
+
 @pytest.mark.parametrize("dtype, width, ff", [(torch.float32, 56, 24), (torch.bfloat16, 64, 40), (torch.bfloat16, 56, 24),
                                              (torch.bfloat16, 128, 96)])
 @pytest.mark.parametrize("rows", [3, 150, 700])
