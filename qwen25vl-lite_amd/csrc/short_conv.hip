@@ -5,29 +5,61 @@
 // of the request's next run and replaced at the end of this one.  x is the float32 residual; the result is
 // written in the run's storage type.
 //
-// Grid (N + R, channel blocks).  Rows below N are tokens: a token that stands at least taps - 1 tokens into
+// Grid (N + R, channel blocks); a thread owns one channel, or four neighbouring ones where 4 divides C.  Rows below N are tokens: a token that stands at least taps - 1 tokens into
 // its run reads only x.  The last R rows are requests: the thread of a channel forms the outputs of the
 // run's first taps - 1 tokens from the old state and then writes the new one, so nobody else reads or
 // writes that channel of the slot in this launch.
 #include "common.h"
 
-template <typename TO>
+// VEC neighbouring channels a thread (4 with C a multiple of 4: 16-byte loads of x and of the state)
+template <int VEC> struct Chan { float v[VEC]; };
+template <int VEC> __device__ __forceinline__ Chan<VEC> ld_chan(const float* p) {
+  Chan<VEC> o;
+  if (VEC == 4) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    o.v[0] = t.x; o.v[VEC > 1 ? 1 : 0] = t.y; o.v[VEC > 2 ? 2 : 0] = t.z; o.v[VEC > 3 ? 3 : 0] = t.w;
+  } else {
+    o.v[0] = *p;
+  }
+  return o;
+}
+template <int VEC> __device__ __forceinline__ void st_chan(float* p, const Chan<VEC>& a) {
+  if (VEC == 4) *reinterpret_cast<float4*>(p) = float4{a.v[0], a.v[VEC > 1 ? 1 : 0], a.v[VEC > 2 ? 2 : 0], a.v[VEC > 3 ? 3 : 0]};
+  else *p = a.v[0];
+}
+template <typename TO, int VEC> __device__ __forceinline__ void st_out(TO* p, const Chan<VEC>& a) {
+  if (VEC == 4 && sizeof(TO) == 2) {            // four bfloat16 values: one 8-byte store (rows of out are C values apart)
+    uint2 o;
+    o.x = (uint32_t)f32_to_bf16(a.v[0]) | ((uint32_t)f32_to_bf16(a.v[VEC > 1 ? 1 : 0]) << 16);
+    o.y = (uint32_t)f32_to_bf16(a.v[VEC > 2 ? 2 : 0]) | ((uint32_t)f32_to_bf16(a.v[VEC > 3 ? 3 : 0]) << 16);
+    *reinterpret_cast<uint2*>(p) = o;
+    return;
+  }
+#pragma unroll
+  for (int u = 0; u < VEC; ++u) stf<TO>(p + u, a.v[u]);
+}
+
+template <typename TO, int VEC>
 __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                          float* __restrict__ state, const int* __restrict__ cu_q,
                                                          const int* __restrict__ req_slots,
                                                          const int* __restrict__ token_req, TO* __restrict__ out, int N,
                                                          int C, int taps) {
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
   if (c >= C) return;
-  const float* wc = w + (size_t)c * taps;
+  const float* wc = w + (size_t)c * taps;      // channel c + u: wc[u * taps + j]
   const int keep = taps - 1;
   if ((int)blockIdx.x < N) {
     const int t = blockIdx.x;
     const int i = t - cu_q[token_req[t]];
     if (i < keep) return;                       // the request's row forms it from the state
-    float acc = x[(size_t)t * C + c];
-    for (int j = 0; j < taps; ++j) acc += wc[j] * x[(size_t)(t - keep + j) * C + c];
-    stf<TO>(out + (size_t)t * C + c, acc);
+    Chan<VEC> acc = ld_chan<VEC>(x + (size_t)t * C + c);
+    for (int j = 0; j < taps; ++j) {
+      const Chan<VEC> v = ld_chan<VEC>(x + (size_t)(t - keep + j) * C + c);
+#pragma unroll
+      for (int u = 0; u < VEC; ++u) acc.v[u] += wc[u * taps + j] * v.v[u];
+    }
+    st_out<TO, VEC>(out + (size_t)t * C + c, acc);
     return;
   }
   const int r = blockIdx.x - N;
@@ -36,19 +68,20 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict
   float* st = state + (size_t)req_slots[r] * keep * C + c;      // st[k * C]: input number k of the kept ones
   const int first = n < keep ? n : keep;
   for (int i = 0; i < first; ++i) {
-    float acc = x[(size_t)(begin + i) * C + c];
+    Chan<VEC> acc = ld_chan<VEC>(x + (size_t)(begin + i) * C + c);
     for (int j = 0; j < taps; ++j) {
       const int src = i - keep + j;             // index into this run; negative: the kept inputs
-      const float v = src >= 0 ? x[(size_t)(begin + src) * C + c] : st[(size_t)(keep + src) * C];
-      acc += wc[j] * v;
+      const Chan<VEC> v = src >= 0 ? ld_chan<VEC>(x + (size_t)(begin + src) * C + c) : ld_chan<VEC>(st + (size_t)(keep + src) * C);
+#pragma unroll
+      for (int u = 0; u < VEC; ++u) acc.v[u] += wc[u * taps + j] * v.v[u];
     }
-    stf<TO>(out + (size_t)(begin + i) * C + c, acc);
+    st_out<TO, VEC>(out + (size_t)(begin + i) * C + c, acc);
   }
   // the last `keep` inputs of (kept inputs, this run); entry k comes from a place behind k, so ascending order
   // never reads what it has overwritten
   for (int k = 0; k < keep; ++k) {
     const int at = n + k;                       // index into (kept inputs, this run)
-    st[(size_t)k * C] = at < keep ? st[(size_t)at * C] : x[(size_t)(begin + at - keep) * C + c];
+    st_chan<VEC>(st + (size_t)k * C, at < keep ? ld_chan<VEC>(st + (size_t)at * C) : ld_chan<VEC>(x + (size_t)(begin + at - keep) * C + c));
   }
 }
 
@@ -62,16 +95,15 @@ extern "C" int qvl_short_conv(const void* x, const void* w, void* state, const v
   if (taps > 1 && (!state || !req_slots)) return QVL_ERR_SHAPE;
   const long long rows = (long long)N + (taps > 1 ? R : 0);
   if (rows > 0x7fffffffll || (C + 255) / 256 > 65535) return QVL_ERR_LIMIT;
-  const dim3 grid((unsigned)rows, (C + 255) / 256);
-  if (out_dtype == 0)
-    hipLaunchKernelGGL(short_conv_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, (const float*)w,
-                       (float*)state, (const int*)cu_q, (const int*)req_slots, (const int*)token_req, (float*)out, N, C,
-                       taps);
-  else if (out_dtype == 1)
-    hipLaunchKernelGGL(short_conv_kernel<bf16_t>, grid, dim3(256), 0, stream, (const float*)x, (const float*)w,
-                       (float*)state, (const int*)cu_q, (const int*)req_slots, (const int*)token_req, (bf16_t*)out, N, C,
-                       taps);
-  else
-    return QVL_ERR_DTYPE;
+  const bool vec = C % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)out & 15) == 0;
+  const int per_block = vec ? 1024 : 256;
+  const dim3 grid((unsigned)rows, (C + per_block - 1) / per_block);
+#define SC_LAUNCH(TO, VEC)                                                                                          \
+  hipLaunchKernelGGL((short_conv_kernel<TO, VEC>), grid, dim3(256), 0, stream, (const float*)x, (const float*)w,     \
+                     (float*)state, (const int*)cu_q, (const int*)req_slots, (const int*)token_req, (TO*)out, N, C, taps)
+  if (out_dtype == 0) { if (vec) SC_LAUNCH(float, 4); else SC_LAUNCH(float, 1); }
+  else if (out_dtype == 1) { if (vec) SC_LAUNCH(bf16_t, 4); else SC_LAUNCH(bf16_t, 1); }
+  else return QVL_ERR_DTYPE;
+#undef SC_LAUNCH
   return qvl_launch_status();
 }

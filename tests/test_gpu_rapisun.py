@@ -110,7 +110,7 @@ def _commit(runner, runs):
         runner.cache.commit(rid, start + n)
 
 
-@pytest.mark.parametrize("width", [5, 72, 1000, 9000])
+@pytest.mark.parametrize("width", [5, 72, 1000, 9000, 20000, 33002])
 @pytest.mark.parametrize("ydtype", [torch.float32, torch.bfloat16])
 def test_layer_norm_adds_into_the_sum(width, ydtype):
     from qwen25vl_lite_amd.ops import rownorm
@@ -136,7 +136,7 @@ def test_layer_norm_adds_into_the_sum(width, ydtype):
     assert torch.allclose(out.cpu().double(), plain.layer_norm(h.double()[rows.long()], w.double(), 1e-5), atol=1e-5)
 
 
-@pytest.mark.parametrize("inter", [3, 88, 2048, 8200])
+@pytest.mark.parametrize("inter", [3, 88, 2048, 8200, 18960, 33000])
 def test_normed_powers(inter):
     from qwen25vl_lite_amd.ops import rownorm
     torch.manual_seed(inter)
@@ -151,13 +151,13 @@ def test_normed_powers(inter):
     assert torch.allclose(got, want, atol=2e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("c", [70, 72, 1100])
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
-def test_short_convolution_across_steps_and_requests(taps, tmp_path):
+def test_short_convolution_across_steps_and_requests(taps, c, tmp_path):
     """One run of 40 tokens against the same tokens in portions (1, 2, 1, 5, ... tokens: shorter and longer than
     the taps) beside another request whose slot is then used again by a third."""
     from qwen25vl_lite_amd.ops.short_conv import short_conv_add
     torch.manual_seed(taps)
-    c = 70
     w = torch.randn(c, taps)
     xs = {rid: torch.randn(n, c) for rid, n in (("p", 40), ("q", 11), ("r", 9))}
     want = {rid: (x.double() + plain.causal_conv(x.double(), w.double())) for rid, x in xs.items()}
