@@ -8,7 +8,7 @@
 //   squared relu   out = max(z, 0)^2
 //
 // A block of 256 threads owns a row.  Rows of up to 256 * 32 values stay in registers between the
-// passes (PER values a thread, the smallest power of two that holds the row); longer rows are read again.
+// passes (PER values, or groups of four values, a thread); longer rows are read again.
 #include "common.h"
 
 #define RN_THREADS 256
@@ -244,7 +244,10 @@ extern "C" int qvl_normed_powers(const void* z, int z_dtype, const void* coeff, 
     else if (per <= 2) NP_LAUNCH(TS, TO, 2, 4);                                                                     \
     else if (per <= 4) NP_LAUNCH(TS, TO, 4, 4);                                                                     \
     else if (per <= 8) NP_LAUNCH(TS, TO, 8, 4);                                                                     \
+    else if (per <= 12) NP_LAUNCH(TS, TO, 12, 4);                                                                   \
     else if (per <= 16) NP_LAUNCH(TS, TO, 16, 4);                                                                   \
+    else if (per <= 20) NP_LAUNCH(TS, TO, 20, 4);                                                                   \
+    else if (per <= 24) NP_LAUNCH(TS, TO, 24, 4);                                                                   \
     else NP_LAUNCH(TS, TO, 32, 4);                                                                                  \
   } else {                                                                                                          \
     const int per = (I + RN_THREADS - 1) / RN_THREADS;                                                              \

@@ -1,12 +1,12 @@
 // A short causal convolution over time on every channel, added to its input:
-//   out[t, c] = x[t, c] + sum_j w[c, j] * x[t - taps + 1 + j, c],   j = 0 .. taps - 1
+//   out[t, c] = x[t, c] + sum_j w[j, c] * x[t - taps + 1 + j, c],   j = 0 .. taps - 1   (w is [taps, C])
 // over the tokens of one request; inputs before the request's first token are zeros.  The last taps - 1
 // inputs of a request are its state (float32 [slots, taps - 1, C], oldest first), read by the first tokens
 // of the request's next run and replaced at the end of this one.  x is the float32 residual; the result is
 // written in the run's storage type.
 //
-// Grid (N + R, channel blocks); a thread owns one channel, or four neighbouring ones where 4 divides C.  Rows below N are tokens: a token that stands at least taps - 1 tokens into
-// its run reads only x.  The last R rows are requests: the thread of a channel forms the outputs of the
+// Grid (N + R, channel blocks); a thread owns one channel, or four neighbouring ones where 4 divides C.
+// Rows below N are tokens: a token that stands at least taps - 1 tokens into its run reads only x.  The last R rows are requests: the thread of a channel forms the outputs of the
 // run's first taps - 1 tokens from the old state and then writes the new one, so nobody else reads or
 // writes that channel of the slot in this launch.
 #include "common.h"
@@ -39,7 +39,8 @@ template <typename TO, int VEC> __device__ __forceinline__ void st_out(TO* p, co
   for (int u = 0; u < VEC; ++u) stf<TO>(p + u, a.v[u]);
 }
 
-template <typename TO, int VEC>
+// MAXT: up to this many taps a token's loads are issued together
+template <typename TO, int VEC, int MAXT>
 __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                          float* __restrict__ state, const int* __restrict__ cu_q,
                                                          const int* __restrict__ req_slots,
@@ -47,17 +48,38 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict
                                                          int C, int taps) {
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
   if (c >= C) return;
-  const float* wc = w + (size_t)c * taps;      // channel c + u: wc[u * taps + j]
+  const float* wc = w + c;                      // tap j of channels c ..: wc[j * C]
   const int keep = taps - 1;
   if ((int)blockIdx.x < N) {
     const int t = blockIdx.x;
     const int i = t - cu_q[token_req[t]];
     if (i < keep) return;                       // the request's row forms it from the state
+    if (taps <= MAXT) {
+      // every load is on its way before the first is used: tap j >= taps reads tap taps - 1 again and counts zero
+      Chan<VEC> xv[MAXT];
+      float wv[VEC][MAXT];
+#pragma unroll
+      for (int j = 0; j < MAXT; ++j) {
+        const int jj = j < taps ? j : keep;
+        xv[j] = ld_chan<VEC>(x + (size_t)(t - keep + jj) * C + c);
+        const Chan<VEC> wj = ld_chan<VEC>(wc + (size_t)jj * C);
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) wv[u][j] = wj.v[u];
+      }
+      Chan<VEC> acc = xv[MAXT - 1];              // x[t]
+#pragma unroll
+      for (int j = 0; j < MAXT; ++j)
+#pragma unroll
+        for (int u = 0; u < VEC; ++u) acc.v[u] += (j < taps ? wv[u][j] : 0.f) * xv[j].v[u];
+      st_out<TO, VEC>(out + (size_t)t * C + c, acc);
+      return;
+    }
     Chan<VEC> acc = ld_chan<VEC>(x + (size_t)t * C + c);
     for (int j = 0; j < taps; ++j) {
       const Chan<VEC> v = ld_chan<VEC>(x + (size_t)(t - keep + j) * C + c);
+      const Chan<VEC> wj = ld_chan<VEC>(wc + (size_t)j * C);
 #pragma unroll
-      for (int u = 0; u < VEC; ++u) acc.v[u] += wc[u * taps + j] * v.v[u];
+      for (int u = 0; u < VEC; ++u) acc.v[u] += wj.v[u] * v.v[u];
     }
     st_out<TO, VEC>(out + (size_t)t * C + c, acc);
     return;
@@ -72,8 +94,9 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict
     for (int j = 0; j < taps; ++j) {
       const int src = i - keep + j;             // index into this run; negative: the kept inputs
       const Chan<VEC> v = src >= 0 ? ld_chan<VEC>(x + (size_t)(begin + src) * C + c) : ld_chan<VEC>(st + (size_t)(keep + src) * C);
+      const Chan<VEC> wj = ld_chan<VEC>(wc + (size_t)j * C);
 #pragma unroll
-      for (int u = 0; u < VEC; ++u) acc.v[u] += wc[u * taps + j] * v.v[u];
+      for (int u = 0; u < VEC; ++u) acc.v[u] += wj.v[u] * v.v[u];
     }
     st_out<TO, VEC>(out + (size_t)(begin + i) * C + c, acc);
   }
@@ -85,7 +108,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict
   }
 }
 
-// x float32 [N, C]; w float32 [C, taps]; state float32 [slots, taps - 1, C] (unused with taps == 1);
+// x float32 [N, C]; w float32 [taps, C] (tap j of every channel side by side); state float32 [slots, taps - 1, C] (unused with taps == 1);
 // cu_q [R + 1], req_slots [R], token_req [N] int32; out [N, C] of out_dtype (0 float32, 1 bfloat16).
 extern "C" int qvl_short_conv(const void* x, const void* w, void* state, const void* cu_q, const void* req_slots,
                               const void* token_req, void* out, int out_dtype, int N, int R, int C, int taps,
@@ -95,11 +118,11 @@ extern "C" int qvl_short_conv(const void* x, const void* w, void* state, const v
   if (taps > 1 && (!state || !req_slots)) return QVL_ERR_SHAPE;
   const long long rows = (long long)N + (taps > 1 ? R : 0);
   if (rows > 0x7fffffffll || (C + 255) / 256 > 65535) return QVL_ERR_LIMIT;
-  const bool vec = C % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)out & 15) == 0;
+  const bool vec = C % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)out & 15) == 0;
   const int per_block = vec ? 1024 : 256;
   const dim3 grid((unsigned)rows, (C + per_block - 1) / per_block);
 #define SC_LAUNCH(TO, VEC)                                                                                          \
-  hipLaunchKernelGGL((short_conv_kernel<TO, VEC>), grid, dim3(256), 0, stream, (const float*)x, (const float*)w,     \
+  hipLaunchKernelGGL((short_conv_kernel<TO, VEC, 4>), grid, dim3(256), 0, stream, (const float*)x, (const float*)w,     \
                      (float*)state, (const int*)cu_q, (const int*)req_slots, (const int*)token_req, (TO*)out, N, C, taps)
   if (out_dtype == 0) { if (vec) SC_LAUNCH(float, 4); else SC_LAUNCH(float, 1); }
   else if (out_dtype == 1) { if (vec) SC_LAUNCH(bf16_t, 4); else SC_LAUNCH(bf16_t, 1); }

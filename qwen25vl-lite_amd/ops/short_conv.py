@@ -16,17 +16,17 @@ _c_int, _c_ptr = ctypes.c_int, ctypes.c_void_p
 
 def short_conv_add(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], cu_q: torch.Tensor,
                    req_slots: torch.Tensor, token_req: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """``out[t] = x[t] + sum_j weight[:, j] * x[t - taps + 1 + j]`` over each request's tokens (``cu_q [R + 1]``
+    """``out[t] = x[t] + sum_j weight[j] * x[t - taps + 1 + j]`` over each request's tokens (``cu_q [R + 1]``
     bounds its run, ``token_req [N]`` names the request of a token), the inputs before a run coming from row
     ``req_slots[r]`` of ``state`` (float32 ``[slots, taps - 1, C]``, oldest first; zeros for a new request), which
-    the run's last inputs replace.  ``x`` float32 ``[N, C]``, ``weight`` float32 ``[C, taps]``; with one tap there
+    the run's last inputs replace.  ``x`` float32 ``[N, C]``, ``weight`` float32 ``[taps, C]`` (a tap's weights of all channels side by side); with one tap there
     is no state.  Returns ``[N, C]`` in ``out_dtype``."""
     _dev(x, weight, state, cu_q, req_slots, token_req)
     _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "x must be contiguous float32 [N, C]")
     n, c = x.shape
-    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[0] == c and weight.is_contiguous(),
-          "the weight must be contiguous float32 [C, taps]")
-    taps = weight.shape[1]
+    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[1] == c and weight.is_contiguous(),
+          "the weight must be contiguous float32 [taps, C]")
+    taps = weight.shape[0]
     for t in (cu_q, req_slots, token_req):
         _need(t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous(), "cu_q, req_slots and token_req must be int32")
     r = req_slots.shape[0]

@@ -17,7 +17,8 @@ class ShortConvolution(Filter):
     before its first token.  The last ``taps - 1`` rows a request has brought are its state (float32
     ``[taps - 1, channels]``, oldest first), so that a sequence may be cut into steps anywhere.
 
-    params: ``channels``, ``taps``.  The weight is ``[channels, taps]`` and is kept in float32.
+    params: ``channels``, ``taps``.  The weight is ``[channels, taps]`` in a checkpoint and is kept in float32 as
+    ``[taps, channels]``, so that neighbouring channels' weights of a tap lie side by side.
     """
 
     graph_safe = True
@@ -37,7 +38,10 @@ class ShortConvolution(Filter):
         return {"weight": ParamSpec((self.channels, self.taps), "vector")}
 
     def load(self, tensors):
-        self.weight = tensors["weight"]
+        self.weight = tensors["weight"].t().contiguous()
+
+    def named_weights(self) -> Dict[str, torch.Tensor]:
+        return {"weight": self.weight.t()}
 
     def forward(self, h: torch.Tensor, step: StepContext, slot: Optional[LayerSlot]) -> torch.Tensor:
         state = slot.state if slot is not None else None

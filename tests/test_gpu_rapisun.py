@@ -178,7 +178,7 @@ def test_short_convolution_across_steps_and_requests(taps, c, tmp_path):
         cu = torch.tensor([0] + list(torch.tensor([n for _, n in runs]).cumsum(0)), dtype=torch.int32).cuda()
         req = torch.cat([torch.full((n,), i, dtype=torch.int32) for i, (_, n) in enumerate(runs)]).cuda()
         sl = torch.tensor([slots[rid] for rid, _ in runs], dtype=torch.int32).cuda()
-        out = short_conv_add(x, w.cuda(), state, cu, sl, req, torch.float32).cpu()
+        out = short_conv_add(x, w.t().contiguous().cuda(), state, cu, sl, req, torch.float32).cpu()
         k = 0
         for rid, n in runs:
             got[rid].append(out[k:k + n])
