@@ -95,7 +95,7 @@ def dazapel_config(layers, size="7b", experts=32, top=6, window=1024, keep_first
             "residual_mult": 0.5, "layers": [{"type": "attention", "mixer": mixer(i), "mlp": mlp} for i in range(int(layers))]}
 
 
-RAPISUN_ORDER = ("hgrn2", "latent", "latent_shared", "hgrn2")
+RAPISUN_ORDER = ("hgrn2", "latent", "hgrn2", "latent_shared")
 
 
 def rapisun_config(layers, size="7b", order=RAPISUN_ORDER, experts=32, top=6, window=1024, kv_rank=192, rot_dim=64):
@@ -118,7 +118,7 @@ def rapisun_config(layers, size="7b", order=RAPISUN_ORDER, experts=32, top=6, wi
             lay = {"type": "hgrn2", "mixer": {"heads": nh, "dim": hd // 2, "vdim": hd}}
         else:
             m = {"heads": nh, "dim": hd, "rot_dim": rot_dim, "vdim": hd, "q_rank": width // 4 // 16 * 16,
-                 "kv_rank": kv_rank, "scale": (hd + rot_dim) ** -0.5, "rot": {"base": 250000.0, "dims": rot_dim},
+                 "kv_rank": kv_rank, "scale": (hd + rot_dim) ** -0.5, "rot": {"base": 100000.0, "dims": rot_dim},
                  "mask": {"size": window}}
             if kind == "latent_shared" and owner is not None:
                 m["kv_from"] = owner
