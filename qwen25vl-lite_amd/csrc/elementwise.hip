@@ -4,29 +4,29 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------
-// Embedding gather: out[n, :] = float32(table[ids[n], :])       (reference text.py:213)
+// Embedding gather: out[n, :] = scale * float32(table[ids[n], :])       (reference text.py:213)
 // ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                    float* __restrict__ out, int H, int V) {
+                                    float* __restrict__ out, int H, int V, float scale) {
   const int n = blockIdx.x;
   int id = ids[n];
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);  // ids are validated on the host; never read outside the table
   const T* row = table + (size_t)id * H;
   float* o = out + (size_t)n * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ldf<T>(row + i);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ldf<T>(row + i) * scale;
 }
 
 extern "C" int qvl_embed_gather(const void* ids, const void* table, void* out, int N, int H, int V, int dtype,
-                                hipStream_t stream) {
+                                float scale, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
   if (H <= 0 || V <= 0) return QVL_ERR_SHAPE;
   if (dtype == 0)
     hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(N), dim3(256), 0, stream, (const int*)ids,
-                       (const float*)table, (float*)out, H, V);
+                       (const float*)table, (float*)out, H, V, scale);
   else if (dtype == 1)
     hipLaunchKernelGGL(embed_gather_kernel<bf16_t>, dim3(N), dim3(256), 0, stream, (const int*)ids,
-                       (const bf16_t*)table, (float*)out, H, V);
+                       (const bf16_t*)table, (float*)out, H, V, scale);
   else
     return QVL_ERR_DTYPE;
   return qvl_launch_status();

@@ -324,7 +324,9 @@ extern "C" int qvl_head_gate(void* o, const void* gate, long long gate_stride, i
 //   head vector a -> a / sqrt(mean(a^2) + eps) * nw (nw = qw for query heads, kw for key heads; a
 //   null weight is a gain of one) -> rotation of the first 2 rot_half channels by the angles whose
 //   cosines and sines are cs[n, f]: pair (2f, 2f+1) if `interleaved`, else (f, f + rot_half).
-//   norm_mode 0: no norm; 1: the norm comes before the rotation; 2: after it.
+//   norm_mode 0: no norm; 1: the norm comes before the rotation; 2: after it; 3: before it and over all
+//   query heads of a token together (and all its key heads together): the two inverse root mean squares
+//   come in `row_rs` [N, 2] (row_inv_rms below forms them) and the weights span all heads' columns.
 //   Queries go to q_out [N, nq hd]; keys into k_cache [pages, nkv, ps, hd] at slots[n]; values
 //   (the key head before norm and rotation, or the value head) into v_cache [pages, nkv, vd, ps].
 // One wave per (token, head); a block holds 4 of them.  hd, vd <= 512.
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     const float* __restrict__ x, long long x_stride, const float* __restrict__ bias, const float* __restrict__ qw,
     const float* __restrict__ kw, const float2* __restrict__ cs, const int* __restrict__ slots, T* __restrict__ q_out,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int N, int nq, int nkv, int hd, int vd, int rot_half, int ps,
-    float eps, int interleaved, int v_from_k, int write_kv, int norm_mode) {
+    float eps, int interleaved, int v_from_k, int write_kv, int norm_mode, const float* __restrict__ row_rs) {
   __shared__ float buf[4][QKN_MAX_HD];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int heads = nq + (write_kv ? (v_from_k ? nkv : 2 * nkv) : 0);
@@ -373,6 +375,10 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
   if (norm_mode == 1) {
     const float rs = 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps);
     for (int c = lane; c < hd; c += 64) mine[c] = nw ? (mine[c] * rs) * nw[c] : mine[c] * rs;
+  } else if (norm_mode == 3) {
+    const float rs = row_rs[2 * (size_t)n + kind];
+    const float* nwh = nw ? nw + (size_t)(kind == 0 ? head : head - nq) * hd : nullptr;
+    for (int c = lane; c < hd; c += 64) mine[c] = nwh ? (mine[c] * rs) * nwh[c] : mine[c] * rs;
   }
   __builtin_amdgcn_wave_barrier();
   T* dst = kind == 0 ? q_out + ((size_t)n * nq + head) * hd
@@ -414,12 +420,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
 extern "C" int qvl_qk_norm_rope_write(const void* x, long long x_stride, const void* bias, const void* qw,
                                       const void* kw, const void* cs, const void* slots, void* q_out, void* k_cache,
                                       void* v_cache, int N, int nq, int nkv, int hd, int vd, int rot_half, int ps,
-                                      float eps, int interleaved, int v_from_k, int write_kv, int norm_mode, int dtype,
-                                      hipStream_t stream) {
+                                      float eps, int interleaved, int v_from_k, int write_kv, int norm_mode,
+                                      const void* row_rs, int dtype, hipStream_t stream) {
   if (N <= 0) return QVL_OK;
   if (nq <= 0 || nkv < 0 || hd <= 0 || vd <= 0 || rot_half < 0 || 2 * rot_half > hd || ps <= 0) return QVL_ERR_SHAPE;
   if (write_kv && (!slots || !k_cache || !v_cache || nkv <= 0)) return QVL_ERR_SHAPE;
-  if (norm_mode < 0 || norm_mode > 2 || (v_from_k && vd != hd)) return QVL_ERR_SHAPE;
+  if (norm_mode < 0 || norm_mode > 3 || (norm_mode == 3 && !row_rs) || (v_from_k && vd != hd)) return QVL_ERR_SHAPE;
   if (hd > QKN_MAX_HD || vd > QKN_MAX_HD) return QVL_ERR_LIMIT;
   const int heads = nq + (write_kv ? (v_from_k ? nkv : 2 * nkv) : 0);
   const long long items = (long long)N * heads;
@@ -428,11 +434,49 @@ extern "C" int qvl_qk_norm_rope_write(const void* x, long long x_stride, const v
   hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(blocks), dim3(256), 0, stream, (const float*)x, x_stride,   \
                      (const float*)bias, (const float*)qw, (const float*)kw, (const float2*)cs, (const int*)slots, \
                      (T*)q_out, (T*)k_cache, (T*)v_cache, N, nq, nkv, hd, vd, rot_half, ps, eps, interleaved,      \
-                     v_from_k, write_kv, norm_mode)
+                     v_from_k, write_kv, norm_mode, (const float*)row_rs)
   if (dtype == 0) LAUNCH(float);
   else if (dtype == 1) LAUNCH(bf16_t);
   else return QVL_ERR_DTYPE;
 #undef LAUNCH
+  return qvl_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Inverse root mean squares of two neighbouring column ranges of every row:
+//   out[n, 0] = 1 / sqrt(mean((x[n, 0 .. c0) + bias)^2) + eps),  out[n, 1] the same over [c0, c0 + c1)
+// (c1 may be 0: then out[n, 1] is 1).  One block per row; the order of the sums depends on the sizes only.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void row_inv_rms_kernel(const float* __restrict__ x, long long x_stride,
+                                                          const float* __restrict__ bias, int c0, int c1, float eps,
+                                                          float* __restrict__ out) {
+  __shared__ float red[17];
+  const size_t n = blockIdx.x;
+  const float* row = x + n * x_stride;
+  float s0 = 0.f, s1 = 0.f;
+  for (int c = threadIdx.x; c < c0; c += blockDim.x) {
+    const float v = row[c] + (bias ? bias[c] : 0.f);
+    s0 += v * v;
+  }
+  for (int c = threadIdx.x; c < c1; c += blockDim.x) {
+    const float v = row[c0 + c] + (bias ? bias[c0 + c] : 0.f);
+    s1 += v * v;
+  }
+  const float t0 = block_sum(s0, red);
+  __syncthreads();
+  const float t1 = c1 > 0 ? block_sum(s1, red) : 0.f;
+  if (threadIdx.x == 0) {
+    out[2 * n] = 1.0f / sqrtf(t0 / (float)c0 + eps);
+    out[2 * n + 1] = c1 > 0 ? 1.0f / sqrtf(t1 / (float)c1 + eps) : 1.0f;
+  }
+}
+
+extern "C" int qvl_row_inv_rms(const void* x, long long x_stride, const void* bias, int c0, int c1, float eps, void* out,
+                               int N, hipStream_t stream) {
+  if (N <= 0) return QVL_OK;
+  if (c0 <= 0 || c1 < 0 || x_stride < (long long)c0 + c1 || !x || !out) return QVL_ERR_SHAPE;
+  hipLaunchKernelGGL(row_inv_rms_kernel, dim3(N), dim3(256), 0, stream, (const float*)x, x_stride, (const float*)bias,
+                     c0, c1, eps, (float*)out);
   return qvl_launch_status();
 }
 

@@ -1,6 +1,6 @@
 """Model specs and the generic decoder.  Importing the package registers the architectures."""
 
-from . import dazapel, gogudra, qwen25vl_text, rapisun  # noqa: F401  (registration)
+from . import dazapel, gogudra, qwen25vl_text, rapisun, rofapel  # noqa: F401  (registration)
 from .decoder import DecoderModel
 from .spec import LayerSpec, ModelSpec, RunEntry
 

@@ -57,6 +57,53 @@ class PassVectors(Part):
         self.weight = tensors["weight"]
 
 
+class PassMix(Part):
+    """``x <- W [x; x0]`` for a matrix ``W [hidden, 2 hidden]``: the running residual sum and the embedding's output
+    of every token, mixed into the sum a pass starts from.  The two halves of ``W`` are kept apart, so nothing is
+    laid side by side at run time, and the half that reads the embedding's output is applied once per step."""
+
+    graph_safe = True
+
+    def __init__(self, hidden: int, dtype, device):
+        super().__init__(dtype, device)
+        self.hidden = int(hidden)
+        self.w_sum: Optional[torch.Tensor] = None     # [hidden, hidden]: the columns that read the running sum
+        self.w_first: Optional[torch.Tensor] = None   # [hidden, hidden]: the columns that read the embedding's output
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.hidden, 2 * self.hidden), "matrix")}
+
+    def load(self, tensors):
+        w = tensors["weight"]
+        self.w_sum = w[:, :self.hidden].contiguous()
+        self.w_first = w[:, self.hidden:].contiguous()
+
+    def named_weights(self) -> Dict[str, torch.Tensor]:
+        return {"weight": torch.cat([self.w_sum, self.w_first], dim=1)}
+
+    def _rounded(self, h: torch.Tensor) -> torch.Tensor:
+        return h if h.dtype == self.dtype else h.to(self.dtype)
+
+    def from_first(self, x0: torch.Tensor) -> torch.Tensor:
+        """float32 ``[N, hidden]``: the embedding's share of every pass's start."""
+        from ..ops.linear import linear
+        return linear(self._rounded(x0), self.w_first, out_dtype=torch.float32)
+
+    def forward(self, stream: ResidualStream, first_share: torch.Tensor) -> ResidualStream:
+        """The stream whose sum is ``w_sum x`` with ``first_share`` waiting to be added (by the next norm)."""
+        from ..ops.gated import residual_add, sandwich_norm
+        from ..ops.linear import linear
+
+        if stream.pending_norm is not None or stream.row_addend is not None:
+            gain, eps_y, factor = stream.pending_norm or (None, 0.0, 1.0)
+            sandwich_norm(stream.h, stream.pending, gain if stream.pending is not None else None, eps_y, factor,
+                          stream.row_addend, None, 0.0, self.dtype)
+        elif stream.pending is not None:
+            residual_add(stream.h, stream.pending)
+        h = linear(self._rounded(stream.h), self.w_sum, out_dtype=torch.float32)
+        return ResidualStream(h if h.is_contiguous() else h.contiguous(), pending=first_share)
+
+
 class DecoderModel:
     """Holds the parts and runs a step over them.  Tensors arrive through :meth:`load_part`."""
 
@@ -75,10 +122,17 @@ class DecoderModel:
             if not spec.pass_vectors_name.endswith(".weight") or spec.pass_vectors_rows <= 0:
                 raise ValueError("pass vectors are a tensor '<name>.weight' with at least one row")
             self.pass_vectors = PassVectors(spec.pass_vectors_rows, spec.hidden_size, dtype, self.device)
+        self.pass_mix: Optional[PassMix] = None
+        if spec.pass_mix_name is not None:
+            if not spec.pass_mix_name.endswith(".weight"):
+                raise ValueError("the pass-mix matrix is a tensor '<name>.weight'")
+            self.pass_mix = PassMix(spec.hidden_size, dtype, self.device)
         for i, entry in enumerate(spec.run):
             if entry.add_vector is not None and not (self.pass_vectors is not None
                                                      and 0 <= entry.add_vector < spec.pass_vectors_rows):
                 raise ValueError(f"run entry {i} adds pass vector {entry.add_vector}, which the model does not have")
+            if entry.mix_input and self.pass_mix is None:
+                raise ValueError(f"run entry {i} mixes the embedding's output in, but the model has no matrix for it")
 
         # The run list: which cache layer and state every mixer of every entry owns.  The lists
         # below have one element per (run entry, mixer of its block), in run order ("places");
@@ -136,6 +190,8 @@ class DecoderModel:
         _collect(self.embedding, _prefix_of(spec.embed_name), self.params)
         if self.pass_vectors is not None:
             _collect(self.pass_vectors, _prefix_of(spec.pass_vectors_name), self.params)
+        if self.pass_mix is not None:
+            _collect(self.pass_mix, _prefix_of(spec.pass_mix_name), self.params)
         for ls, block in zip(spec.layers, self.blocks):
             _collect(block, ls.prefix, self.params)
         _collect(self.final_norm, spec.final_norm_prefix, self.params)
@@ -150,7 +206,8 @@ class DecoderModel:
         """True if every part may run under HIP graph capture."""
         def safe(part) -> bool:
             return part.graph_safe and all(safe(s) for s in part.sub_parts().values())
-        return all(safe(b) for b in self.blocks) and safe(self.final_norm) and safe(self.embedding) and safe(self.head_part)
+        return (all(safe(b) for b in self.blocks) and safe(self.final_norm) and safe(self.embedding)
+                and safe(self.head_part))
 
 
     def cache_groups(self) -> List[CacheGroupSpec]:
@@ -214,7 +271,12 @@ class DecoderModel:
         if not self._has_weights:
             raise RuntimeError("the model has no weights yet")
         stream = ResidualStream(self.embedding.forward(step.token_ids, step))
+        first_share = None
+        if self.pass_mix is not None and any(e.mix_input for e in self.spec.run):
+            first_share = self.pass_mix.from_first(stream.h)     # before any layer changes the sum in place
         for entry, slot in zip(self.spec.run, slots):
+            if entry.mix_input:
+                stream = self.pass_mix.forward(stream, first_share)
             if entry.add_vector is not None:
                 if stream.row_addend is not None:
                     raise RuntimeError("a block left a pass vector unadded: its first norm must fold the stream")

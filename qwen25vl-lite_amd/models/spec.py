@@ -36,6 +36,9 @@ class RunEntry:
     # a row of the model's pass vectors that is added to every token's residual sum right before
     # this entry's layer runs
     add_vector: Optional[int] = None
+    # True: right before this entry's layer runs (and before ``add_vector``), every token's residual sum x
+    # becomes ``W [x; x0]``, ``x0`` being what the embedding gave for the token and ``W`` the model's pass-mix matrix
+    mix_input: bool = False
 
 
 @dataclass
@@ -63,3 +66,6 @@ class ModelSpec:
     # of a tensor ``[rows, hidden]`` and its number of rows; None: the model has none
     pass_vectors_name: Optional[str] = None
     pass_vectors_rows: int = 0
+    # the matrix ``[hidden, 2 hidden]`` of the run entries with ``mix_input`` (columns of the running sum first,
+    # then those of the embedding's output): the canonical name of the tensor; None: the model has none
+    pass_mix_name: Optional[str] = None

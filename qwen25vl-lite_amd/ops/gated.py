@@ -13,7 +13,8 @@ import torch
 
 from .kernels import _check, _dev, _fn, _need, _ptr, _stream, dtype_code
 
-__all__ = ["residual_add", "gated_act", "softcap_", "group_norm_gate", "head_gate_", "qk_norm_rope_write", "sandwich_norm"]
+__all__ = ["residual_add", "gated_act", "softcap_", "group_norm_gate", "head_gate_", "qk_norm_rope_write", "sandwich_norm",
+           "row_inv_rms"]
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 GATE_ACTS = {None: 0, "sigmoid": 1, "silu": 2}
@@ -101,6 +102,21 @@ def head_gate_(o: torch.Tensor, gate: torch.Tensor, num_heads: int) -> torch.Ten
     return o
 
 
+def row_inv_rms(x: torch.Tensor, first: int, second: int, eps: float, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 ``[N, 2]``: ``1 / sqrt(mean(x[n, :first]^2) + eps)`` and the same over the next ``second`` columns
+    (1 if there are none) of float32 ``x [N, >= first + second]``, ``bias`` added to the columns first."""
+    _dev(x, bias)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1 and first > 0 and second >= 0
+          and x.shape[1] >= first + second, "x must be float32 [N, at least the two ranges' columns]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.dim() == 1 and bias.shape[0] >= first + second
+                           and bias.is_contiguous()), "the bias must be float32 over the ranges' columns")
+    out = torch.empty((x.shape[0], 2), dtype=torch.float32, device=x.device)
+    fn = _fn("gated", "qvl_row_inv_rms", [_c_ptr, _c_ll, _c_ptr, _c_int, _c_int, _c_float, _c_ptr, _c_int, _c_ptr])
+    _check(fn(_ptr(x), x.stride(0), _ptr(bias), int(first), int(second), float(eps), _ptr(out), x.shape[0], _stream()),
+           "row_inv_rms")
+    return out
+
+
 def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
                        cs: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                        v_cache: Optional[torch.Tensor], num_q_heads: int, num_kv_heads: int, head_dim: int,
@@ -109,7 +125,8 @@ def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: 
                        value_dim: Optional[int] = None) -> torch.Tensor:
     """Per head: ``bias`` (float32 over all columns, or None) is added; RMS norm over the head
     (``norm`` ``"before"`` or ``"after"`` the rotation, None: no norm; weights ``q_norm`` / ``k_norm``
-    of ``[head_dim]``, None: a gain of one); rotation by the angles whose ``(cos, sin)`` are
+    of ``[head_dim]``, None: a gain of one; ``norm`` ``"whole"``: before the rotation and over all query heads of a
+    token at once, and over all its key heads at once, with weights of ``[heads head_dim]``); rotation by the angles whose ``(cos, sin)`` are
     ``cs [N, rot/2, 2]``: pairs ``(2f, 2f+1)`` if ``interleaved``, else ``(f, f + rot/2)``.  Rotated
     queries are returned; rotated keys and the values go into the page slots (``slots`` None:
     queries only).  ``x`` is float32 ``[N, >= nq hd + nkv hd (+ nkv vd)]``: query heads, key heads, and value
@@ -123,11 +140,16 @@ def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: 
     cols = nq * hd + ((nkv * hd + (0 if values_are_keys else nkv * vd)) if write else 0)
     _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] >= cols and x.stride(1) == 1,
           "x must be float32 [N, at least the heads' columns]")
-    _need(norm in (None, "before", "after"), "the norm stands before or after the rotation, or is None")
+    _need(norm in (None, "before", "after", "whole"), "the norm stands before or after the rotation, spans the whole "
+          "projection, or is None")
     _need(not (values_are_keys and vd != hd), "keys that are their own values have the keys' width")
-    for w in (q_norm, k_norm):
-        _need(w is None or (w.dtype == torch.float32 and w.shape == (hd,) and w.is_contiguous()),
-              "a head norm's weight must be float32 [head_dim]")
+    for w, heads in ((q_norm, nq), (k_norm, nkv)):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == ((heads * hd,) if norm == "whole" else (hd,))
+                            and w.is_contiguous()),
+              "a head norm's weight must be float32 [head_dim], a whole projection's [heads head_dim]")
+    row_rs = None
+    if norm == "whole":
+        row_rs = row_inv_rms(x, nq * hd, nkv * hd if write else 0, eps, bias)
     _need(bias is None or (bias.dtype == torch.float32 and bias.dim() == 1 and bias.shape[0] >= cols
                            and bias.is_contiguous()), "the bias must be float32 over the heads' columns")
     _need(cs.dtype == torch.float32 and cs.dim() == 3 and cs.is_contiguous() and cs.shape[0] >= n
@@ -143,11 +165,12 @@ def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: 
     q_out = torch.empty((n, nq * hd), dtype=out_dtype, device=x.device)
     fn = _fn("gated", "qvl_qk_norm_rope_write",
              [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
-              _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr])
+              _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr])
     _check(fn(_ptr(x), x.stride(0), _ptr(bias), _ptr(q_norm), _ptr(k_norm), _ptr(cs), _ptr(slots), _ptr(q_out),
               _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, n, nq, nkv, hd, vd, cs.shape[1],
               int(page_size), float(eps), int(interleaved), int(values_are_keys), int(write),
-              {None: 0, "before": 1, "after": 2}[norm], dtype_code(out_dtype), _stream()), "qk_norm_rope_write")
+              {None: 0, "before": 1, "after": 2, "whole": 3}[norm], _ptr(row_rs), dtype_code(out_dtype), _stream()),
+           "qk_norm_rope_write")
     return q_out
 
 

@@ -82,8 +82,9 @@ def _need(cond: bool, msg: str) -> None:
 
 
 # --------------------------------------------------------------------------------------------
-def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``out[n] = float32(table[ids[n]])`` — the residual stream starts in float32."""
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None,
+                 scale: float = 1.0) -> torch.Tensor:
+    """``out[n] = scale * float32(table[ids[n]])`` — the residual stream starts in float32."""
     _dev(ids, table, out)
     _need(ids.dtype == torch.int32 and ids.dim() == 1 and ids.is_contiguous(), "ids must be contiguous int32 [N]")
     _need(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [V, H]")
@@ -91,8 +92,9 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Ten
     if out is None:
         out = torch.empty((n, h), dtype=torch.float32, device=table.device)
     _need(out.dtype == torch.float32 and out.shape == (n, h) and out.is_contiguous(), "out must be float32 [N, H]")
-    fn = _fn("elementwise", "qvl_embed_gather", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr])
-    _check(fn(_ptr(ids), _ptr(table), _ptr(out), n, h, v, dtype_code(table.dtype), _stream()), "embed_gather")
+    fn = _fn("elementwise", "qvl_embed_gather", [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr])
+    _check(fn(_ptr(ids), _ptr(table), _ptr(out), n, h, v, dtype_code(table.dtype), float(scale), _stream()),
+           "embed_gather")
     return out
 
 

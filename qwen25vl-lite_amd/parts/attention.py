@@ -15,7 +15,8 @@ import torch
 from ..ops import kernels, skinny
 from ..ops.attention import paged_attention
 from ..ops.linear import NormedRows, linear, linear_into
-from .base import (CacheNeed, LayerSlot, Mixer, ParamSpec, PartSpec, StepContext, build_part, register_part)
+from .base import (CacheNeed, LayerSlot, Mixer, ParamSpec, PartSpec, StateNeed, StepContext, build_part,
+                   register_part)
 
 # 33 to 48 rows: the projection cut along its inner size (slabs) and the rotation's kernel behind it beat the
 # fused kernel on teams of blocks (7B sizes: a step of 33 rows 4.14 ms against 4.24, of 48 rows 4.34 against 4.39,
@@ -44,8 +45,14 @@ class PagedAttention(Mixer):
     to every later token; their rotation and their distance to a query are those of where they stand),
     ``element_gate`` (channel ``c`` of the heads' joined output is scaled by ``sigmoid(g_c)``, ``g`` a
     projection of ``[heads value_dim, hidden]``),
-    ``out_bias`` (the output projection has a bias).  Any of these except the last takes the
-    projection through float32 and one kernel that norms, rotates and writes the cache."""
+    ``out_bias`` (the output projection has a bias), ``qk_norm_scope`` (``"head"``, the default, or ``"whole"``: one
+    RMS norm over all of a token's query heads together and one over all its key heads, before the rotation,
+    with weights of ``[heads head_dim]``), ``conv_taps`` (a number: the projected queries and keys pass a causal
+    convolution over time, ``y_t = sum_j w[:, j] u_(t - taps + 1 + j)`` per channel with weights ``q_conv`` /
+    ``k_conv`` of ``[channels, taps]``, before norm and rotation; keys that are their own values are taken behind
+    it; a request's last ``taps - 1`` projected rows are its state), ``sinks`` (True: a tensor ``sink [heads]``
+    whose ``exp`` joins each head's softmax denominator).  Any of these except the output bias and the sinks
+    takes the projection through float32 and one kernel that norms, rotates and writes the cache."""
 
     graph_safe = True
     takes_lazy_norm = True
@@ -69,6 +76,9 @@ class PagedAttention(Mixer):
         self.head_gate = bool(params.get("head_gate", False))
         self.element_gate = bool(params.get("element_gate", False))
         self.out_bias = bool(params.get("out_bias", False))
+        self.qk_norm_scope = str(params.get("qk_norm_scope", "head"))
+        self.conv_taps = int(params.get("conv_taps") or 0)
+        self.has_sinks = bool(params.get("sinks", False))
         self.vd = int(params.get("value_dim") or self.hd)
         self.keep_first = int(params.get("keep_first") or 0) if self.window else 0
         if self.qk_norm_where not in ("before", "after"):
@@ -79,9 +89,18 @@ class PagedAttention(Mixer):
             raise ValueError("keys that are their own values have the keys' width")
         if self.keep_first < 0:
             raise ValueError("keep_first cannot be negative")
+        if self.qk_norm_scope not in ("head", "whole"):
+            raise ValueError("qk_norm_scope is 'head' or 'whole'")
+        if self.qk_norm_scope == "whole" and (self.qk_norm_eps is None or self.qk_norm_where != "before"
+                                              or not self.qk_norm_weights):
+            raise ValueError("a norm over the whole projection stands before the rotation and has weights")
+        if self.conv_taps and not (self.values_are_keys and not self.qkv_bias):
+            raise ValueError("the convolution on queries and keys is built for keys that are their own values, "
+                             "without biases")
         names = dict(params.get("names") or {})
         self.names = {k: names.get(k, d) for k, d in (("q", "q_proj"), ("k", "k_proj"), ("v", "v_proj"), ("o", "o_proj"),
-                                                      ("g", "g_proj"), ("q_norm", "q_norm"), ("k_norm", "k_norm"))}
+                                                      ("g", "g_proj"), ("q_norm", "q_norm"), ("k_norm", "k_norm"),
+                                                      ("q_conv", "q_conv"), ("k_conv", "k_conv"), ("sink", "sink"))}
         self.q_norm: Optional[torch.Tensor] = None
         self.k_norm: Optional[torch.Tensor] = None
         if self.nq % self.nkv:
@@ -90,15 +109,27 @@ class PagedAttention(Mixer):
         self.position = build_part("position", pos, dtype, device)
         self.interleaved = bool(getattr(self.position, "interleaved", False))
         self.normed_path = (self.qk_norm_eps is not None or self.values_are_keys or self.head_gate
-                            or self.element_gate or self.interleaved or self.vd != self.hd)
+                            or self.element_gate or self.interleaved or self.vd != self.hd or bool(self.conv_taps))
         self.gate_rows = self.nq if self.head_gate else (self.nq * self.vd if self.element_gate else 0)
         self.w_in: Optional[torch.Tensor] = None
         self.b_in: Optional[torch.Tensor] = None
         self.w_out: Optional[torch.Tensor] = None
         self.b_out: Optional[torch.Tensor] = None
+        self.w_conv: Optional[torch.Tensor] = None      # float32 [taps, convolved channels]
+        self.sink: Optional[torch.Tensor] = None
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(self.nkv, self.hd, self.window, self.keep_first, None if self.vd == self.hd else self.vd)
+
+    @property
+    def conv_channels(self) -> int:
+        """Columns of the stacked projection that pass the convolution: the queries' and the keys'."""
+        return (self.nq + (0 if self.kv_shared else self.nkv)) * self.hd if self.conv_taps else 0
+
+    def state_need(self) -> Optional[StateNeed]:
+        if self.conv_taps > 1:
+            return StateNeed((self.conv_taps - 1, self.conv_channels), torch.float32)
+        return None
 
     def _projections(self):
         """``(role, rows)`` of the matrices stacked into the input product, in order."""
@@ -117,10 +148,19 @@ class PagedAttention(Mixer):
         if self.qkv_bias:
             for role, rows in self._projections():
                 specs[f"{n[role]}.bias"] = ParamSpec((rows,), "vector")
-        if self.qk_norm_eps is not None and self.qk_norm_weights:
-            specs[f"{n['q_norm']}.weight"] = ParamSpec((self.hd,), "vector", init="around_one")
+        if self.conv_taps:
+            specs[f"{n['q_conv']}.weight"] = ParamSpec((self.nq * self.hd, self.conv_taps), "vector")
             if not self.kv_shared:
-                specs[f"{n['k_norm']}.weight"] = ParamSpec((self.hd,), "vector", init="around_one")
+                specs[f"{n['k_conv']}.weight"] = ParamSpec((self.nkv * self.hd, self.conv_taps), "vector")
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
+            whole = self.qk_norm_scope == "whole"
+            specs[f"{n['q_norm']}.weight"] = ParamSpec((self.nq * self.hd if whole else self.hd,), "vector",
+                                                       init="around_one")
+            if not self.kv_shared:
+                specs[f"{n['k_norm']}.weight"] = ParamSpec((self.nkv * self.hd if whole else self.hd,), "vector",
+                                                           init="around_one")
+        if self.has_sinks:
+            specs[f"{n['sink']}.weight"] = ParamSpec((self.nq,), "vector")
         if self.gate_rows:
             specs[f"{n['g']}.weight"] = ParamSpec((self.gate_rows, self.hidden))
         specs[f"{n['o']}.weight"] = ParamSpec((self.hidden, self.nq * self.vd))
@@ -145,6 +185,13 @@ class PagedAttention(Mixer):
         if self.qk_norm_eps is not None and self.qk_norm_weights:
             self.q_norm = tensors[f"{n['q_norm']}.weight"]
             self.k_norm = tensors.get(f"{n['k_norm']}.weight")
+        if self.conv_taps:
+            # kept tap-major: neighbouring channels' weights of a tap lie side by side
+            taps = [tensors[f"{n['q_conv']}.weight"]]
+            if not self.kv_shared:
+                taps.append(tensors[f"{n['k_conv']}.weight"])
+            self.w_conv = torch.cat(taps, dim=0).t().contiguous()
+        self.sink = tensors.get(f"{n['sink']}.weight")
 
     def named_weights(self) -> Dict[str, torch.Tensor]:
         """Views of the stacked tensors under their checkpoint names."""
@@ -163,6 +210,12 @@ class PagedAttention(Mixer):
             out[f"{n['q_norm']}.weight"] = self.q_norm
         if self.k_norm is not None:
             out[f"{n['k_norm']}.weight"] = self.k_norm
+        if self.w_conv is not None:
+            out[f"{n['q_conv']}.weight"] = self.w_conv[:, :self.nq * self.hd].t()
+            if not self.kv_shared:
+                out[f"{n['k_conv']}.weight"] = self.w_conv[:, self.nq * self.hd:].t()
+        if self.sink is not None:
+            out[f"{n['sink']}.weight"] = self.sink
         out[f"{n['o']}.weight"] = self.w_out
         return out
 
@@ -181,7 +234,7 @@ class PagedAttention(Mixer):
         if q is None:
             q = self._project(x, step, group, slot, write, inv_freq, freq_row)
         o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale,
-                            keep_first=self.keep_first)
+                            keep_first=self.keep_first, sinks=self.sink)
         return self._output(o, step)
 
     def _output(self, o: torch.Tensor, step: StepContext):
@@ -199,14 +252,21 @@ class PagedAttention(Mixer):
 
         proj = linear(x, self.w_in, out_dtype=torch.float32)     # the bias is added by the kernel that norms
         cs = self._rotation_table(step, inv_freq, freq_row, proj.shape[0])
+        heads_in = proj
+        if self.conv_taps:
+            from ..ops.short_conv import short_conv
+            if self.conv_taps > 1 and slot.state is None:
+                raise RuntimeError("a convolution with more than one tap needs a state slot")
+            heads_in = short_conv(proj[:, :self.conv_channels], self.w_conv, slot.state, step.cu_q, step.req_slots,
+                                  step.token_req, torch.float32)
+        norm = None if self.qk_norm_eps is None else ("whole" if self.qk_norm_scope == "whole" else self.qk_norm_where)
         q = gated.qk_norm_rope_write(
-            proj, self.q_norm, self.k_norm, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0, cs,
+            heads_in, self.q_norm, self.k_norm, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0, cs,
             group.slot_mapping if write else None, slot.k_cache if write else None, slot.v_cache if write else None,
             self.nq, self.nkv, self.hd, group.page_size, self.dtype, interleaved=self.interleaved,
-            values_are_keys=self.values_are_keys, norm=None if self.qk_norm_eps is None else self.qk_norm_where,
-            bias=self.b_in, value_dim=self.vd)
+            values_are_keys=self.values_are_keys, norm=norm, bias=self.b_in, value_dim=self.vd)
         o = paged_attention(q, slot.k_cache, slot.v_cache, group.block_table, step, self.nq, self.window, self.scale,
-                            keep_first=self.keep_first)
+                            keep_first=self.keep_first, sinks=self.sink)
         if self.gate_rows:
             # one gate per head, or one per element (a "head" of one channel)
             at = self.w_in.shape[0] - self.gate_rows

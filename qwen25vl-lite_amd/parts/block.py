@@ -46,10 +46,12 @@ class PreNormBlock(Block):
 
 
 class ParallelBlock(Block):
-    """``x = norm(h); h += mixer(x) + ffn(x)``: one norm, both sublayers read its output.
+    """``x = norm(h); h += mixer(x) + ffn(x)``: one norm, both sublayers read its output; or, with a second
+    norm, ``h += mixer(norm(h)) + ffn(norm2(h))``, both norms of the same ``h``.
 
     params: ``norm``, ``mixer`` (:class:`PartSpec` each), ``ffn`` (a :class:`PartSpec`, or None
-    for a layer without a feed-forward) and ``names``, the checkpoint sub-name of each.  The
+    for a layer without a feed-forward), ``norm2`` (a :class:`PartSpec` or absent: the feed-forward reads the
+    first norm's rows) and ``names``, the checkpoint sub-name of each.  The
     normalised rows are computed before either sublayer runs, so a sublayer's last product may add
     into ``h`` in place; what a sublayer returns instead is added in float32, the first result by a
     kernel of its own, the last one by the next norm's kernel.
@@ -62,18 +64,24 @@ class ParallelBlock(Block):
         self.norm = build_part("norm", params["norm"], dtype, device)
         self.mixer = build_part("mixer", params["mixer"], dtype, device)
         self.ffn: Optional[Part] = None if params.get("ffn") is None else build_part("ffn", params["ffn"], dtype, device)
+        self.norm2: Optional[Part] = None
+        if self.ffn is not None and params.get("norm2") is not None:
+            self.norm2 = build_part("norm", params["norm2"], dtype, device)
         self.names: Dict[str, str] = dict(params["names"])
 
     def sub_parts(self) -> Dict[str, Part]:
         parts = {self.names["norm"]: self.norm, self.names["mixer"]: self.mixer}
         if self.ffn is not None:
             parts[self.names["ffn"]] = self.ffn
+        if self.norm2 is not None:
+            parts[self.names["norm2"]] = self.norm2
         return parts
 
     def forward(self, stream: ResidualStream, step: StepContext, slot: LayerSlot) -> ResidualStream:
         from ..ops.gated import residual_add
 
         x = self.norm.forward(stream)        # never lazily: h changes before the second reader would look
+        x2 = x if self.norm2 is None else self.norm2.forward(stream)   # the sum is folded: this one only norms
         step.residual = stream.h
         y = self.mixer.forward(x, step, slot)
         if self.ffn is None:
@@ -81,7 +89,7 @@ class ParallelBlock(Block):
         else:
             if y is not None:
                 residual_add(stream.h, y)
-            stream.pending = self.ffn.forward(x, step)
+            stream.pending = self.ffn.forward(x2, step)
         step.residual = None
         return stream
 

@@ -28,14 +28,16 @@ __all__ = ["LatentAttention"]
 
 class LatentAttention(Mixer):
     """params: ``hidden_size``, ``num_heads``, ``head_dim`` (a head's unrotated query/key channels), ``rot_dim``
-    (its rotated ones), ``value_dim``, ``q_rank`` and ``kv_rank`` (the latents' sizes), ``scale`` (None:
+    (its rotated ones), ``value_dim``, ``q_rank`` and ``kv_rank`` (the latents' sizes; ``q_rank`` None: the queries
+    are one projection ``q`` of the mixer's input and pass no latent), ``scale`` (None:
     ``(head_dim + rot_dim) ** -0.5``), ``eps`` (of the latents' RMS norms), ``window`` (None: all keys; a number:
     a query at index i sees keys j with ``0 <= i - j < window``), ``retain`` (how many keys back pages are kept,
     None: all; default ``window``; a layer whose cache another layer with a longer window reads keeps more than
     it sees), ``sinks`` (True: a tensor ``sink [heads]`` whose ``exp`` joins each head's softmax denominator),
     ``position`` (a :class:`PartSpec` of category ``position`` for the ``rot_dim`` rotated channels), ``kv_shared``
     (True: no key/value down projection; the layer reads the latents another layer cached, with up projections
-    of its own), ``names`` (``dq``, ``dq_norm``, ``uq``, ``dkv``, ``dkv_norm``, ``uk``, ``uv``, ``sink``, ``o``).
+    of its own), ``names`` (``dq``, ``dq_norm``, ``uq``, ``q``, ``dkv``, ``dkv_norm``, ``uk``, ``uv``, ``sink``, ``o``).  The
+    position encoding says whether rotated channels are paired in halves or as neighbours (``interleaved``).
 
     The down projections are one stacked product left in float32; the norms, the rotation's angles, the scores
     and the softmax are float32; the latents in the cache, the queries and the attended latents are in the run
@@ -50,9 +52,10 @@ class LatentAttention(Mixer):
         self.dim = int(params["head_dim"])
         self.rot_dim = int(params["rot_dim"])
         self.vdim = int(params["value_dim"])
-        self.q_rank = int(params["q_rank"])
+        self.q_rank = int(params["q_rank"]) if params.get("q_rank") is not None else 0   # 0: queries pass no latent
         self.kv_rank = int(params["kv_rank"])
-        if min(self.heads, self.dim, self.vdim, self.q_rank, self.kv_rank) <= 0 or self.rot_dim < 0:
+        if min(self.heads, self.dim, self.vdim, self.kv_rank) <= 0 or self.rot_dim < 0 or self.q_rank < 0 \
+                or (params.get("q_rank") is not None and self.q_rank == 0):
             raise ValueError("a latent attention's sizes must be positive (rot_dim may be 0)")
         scale = params.get("scale")
         self.scale = float(scale) if scale is not None else (self.dim + self.rot_dim) ** -0.5
@@ -66,13 +69,14 @@ class LatentAttention(Mixer):
         self.kv_shared = bool(params.get("kv_shared", False))
         self.has_sinks = bool(params.get("sinks", False))
         names = dict(params.get("names") or {})
-        self.names = {k: names.get(k, k) for k in ("dq", "dq_norm", "uq", "dkv", "dkv_norm", "uk", "uv", "sink", "o")}
+        self.names = {k: names.get(k, k) for k in ("dq", "dq_norm", "uq", "q", "dkv", "dkv_norm", "uk", "uv", "sink", "o")}
         pos: Optional[PartSpec] = params.get("position")
         self.position = build_part("position", pos, dtype, device) if pos is not None and self.rot_dim else None
+        self.interleaved = bool(getattr(self.position, "interleaved", False))
         self.w_down: Optional[torch.Tensor] = None      # [q_rank (+ kv_rank + rot_dim), hidden]
         self.q_norm: Optional[torch.Tensor] = None
         self.kv_norm: Optional[torch.Tensor] = None
-        self.w_uq: Optional[torch.Tensor] = None        # [heads (dim + rot_dim), q_rank]
+        self.w_uq: Optional[torch.Tensor] = None        # [heads (dim + rot_dim), q_rank]; without a query latent [.., hidden]
         self.w_uk_t: Optional[torch.Tensor] = None      # [heads, kv_rank, dim]: Uk_h^T, the matrix that carries a query over
         self.w_uv: Optional[torch.Tensor] = None        # [heads, vdim, kv_rank]
         self.sink: Optional[torch.Tensor] = None
@@ -87,9 +91,12 @@ class LatentAttention(Mixer):
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         n, h = self.names, self.heads
-        specs = {f"{n['dq']}.weight": ParamSpec((self.q_rank, self.hidden)),
-                 f"{n['dq_norm']}.weight": ParamSpec((self.q_rank,), "vector", init="around_one"),
-                 f"{n['uq']}.weight": ParamSpec((h * (self.dim + self.rot_dim), self.q_rank))}
+        if self.q_rank:
+            specs = {f"{n['dq']}.weight": ParamSpec((self.q_rank, self.hidden)),
+                     f"{n['dq_norm']}.weight": ParamSpec((self.q_rank,), "vector", init="around_one"),
+                     f"{n['uq']}.weight": ParamSpec((h * (self.dim + self.rot_dim), self.q_rank))}
+        else:
+            specs = {f"{n['q']}.weight": ParamSpec((h * (self.dim + self.rot_dim), self.hidden))}
         if not self.kv_shared:
             specs[f"{n['dkv']}.weight"] = ParamSpec((self.kv_rank + self.rot_dim, self.hidden))
             specs[f"{n['dkv_norm']}.weight"] = ParamSpec((self.kv_rank,), "vector", init="around_one")
@@ -102,13 +109,13 @@ class LatentAttention(Mixer):
 
     def load(self, tensors):
         n = self.names
-        mats = [tensors[f"{n['dq']}.weight"]]
+        mats = [tensors[f"{n['dq']}.weight"]] if self.q_rank else []
         if not self.kv_shared:
             mats.append(tensors[f"{n['dkv']}.weight"])
             self.kv_norm = tensors[f"{n['dkv_norm']}.weight"]
-        self.w_down = torch.cat(mats, dim=0).contiguous()
-        self.q_norm = tensors[f"{n['dq_norm']}.weight"]
-        self.w_uq = tensors[f"{n['uq']}.weight"]
+        self.w_down = torch.cat(mats, dim=0).contiguous() if mats else None
+        self.q_norm = tensors.get(f"{n['dq_norm']}.weight")
+        self.w_uq = tensors[f"{n['uq' if self.q_rank else 'q']}.weight"]
         self.w_uk_t = tensors[f"{n['uk']}.weight"].view(self.heads, self.dim, self.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = tensors[f"{n['uv']}.weight"].view(self.heads, self.vdim, self.kv_rank)
         self.sink = tensors.get(f"{n['sink']}.weight")
@@ -116,9 +123,13 @@ class LatentAttention(Mixer):
 
     def named_weights(self) -> Dict[str, torch.Tensor]:
         n = self.names
-        out = {f"{n['dq']}.weight": self.w_down[:self.q_rank], f"{n['dq_norm']}.weight": self.q_norm,
-               f"{n['uq']}.weight": self.w_uq, f"{n['uk']}.weight": self.w_uk_t.transpose(1, 2).reshape(-1, self.kv_rank),
+        out = {f"{n['uk']}.weight": self.w_uk_t.transpose(1, 2).reshape(-1, self.kv_rank),
                f"{n['uv']}.weight": self.w_uv.reshape(-1, self.kv_rank), f"{n['o']}.weight": self.w_out}
+        if self.q_rank:
+            out.update({f"{n['dq']}.weight": self.w_down[:self.q_rank], f"{n['dq_norm']}.weight": self.q_norm,
+                        f"{n['uq']}.weight": self.w_uq})
+        else:
+            out[f"{n['q']}.weight"] = self.w_uq
         if not self.kv_shared:
             out[f"{n['dkv']}.weight"] = self.w_down[self.q_rank:]
             out[f"{n['dkv_norm']}.weight"] = self.kv_norm
@@ -147,13 +158,17 @@ class LatentAttention(Mixer):
         group = step.groups[slot.group]
         n, h, r, rot = x.shape[0], self.heads, self.kv_rank, self.rot_dim
         cs = self._rotation_table(step, n)
-        down = linear(x, self.w_down, out_dtype=torch.float32)
-        if self.kv_shared:
-            cq = latent.latent_down(down, self.q_rank, self.q_norm, self.eps, self.dtype)
-        else:
-            cq = latent.latent_down(down, self.q_rank, self.q_norm, self.eps, self.dtype, kv_rank=r, rot_dim=rot,
-                                    kv_norm=self.kv_norm, cs=cs, slots=group.slot_mapping, k_cache=slot.k_cache,
-                                    v_cache=slot.v_cache)
+        cq = x
+        if self.w_down is not None:
+            down = linear(x, self.w_down, out_dtype=torch.float32)
+            if self.kv_shared:
+                cq = latent.latent_down(down, self.q_rank, self.q_norm, self.eps, self.dtype)
+            else:
+                cq = latent.latent_down(down, self.q_rank, self.q_norm, self.eps, self.dtype, kv_rank=r, rot_dim=rot,
+                                        kv_norm=self.kv_norm, cs=cs, slots=group.slot_mapping, k_cache=slot.k_cache,
+                                        v_cache=slot.v_cache, interleaved=self.interleaved)
+            if not self.q_rank:
+                cq = x                      # the queries are a projection of the mixer's input itself
         q = linear(cq, self.w_uq)
         q = q if q.is_contiguous() else q.contiguous()
         # the query in the latent's space, head by head: [N, heads, kv_rank | rot_dim]
@@ -163,7 +178,7 @@ class LatentAttention(Mixer):
             by_head = step.per_pass[("pairs_by_head", h)] = moe_ops.pairs_by_column(n, h, x.device)
         moe_ops.expert_products(q.view(n * h, self.dim + rot)[:, :self.dim], self.w_uk_t, *by_head, n * h, 1, self.dtype,
                                 out=q_lat.view(n * h, r + rot)[:, :r])
-        latent.latent_query_rotate_(q, h, self.dim, rot, r, cs, q_lat)
+        latent.latent_query_rotate_(q, h, self.dim, rot, r, cs, q_lat, interleaved=self.interleaved)
         o_lat = paged_attention(q_lat.view(n, h * (r + rot)), slot.k_cache, slot.v_cache, group.block_table, step, h,
                                 self.window, self.scale, sinks=self.sink)
         o = moe_ops.expert_products(o_lat.view(n * h, r), self.w_uv, *by_head, n * h, 1, self.dtype)

@@ -15,7 +15,8 @@ __all__ = ["SwiGLU", "ClampedGatedFF", "PlainFF"]
 class SwiGLU(FeedForward):
     """``down(silu(gate(x)) * up(x))`` without biases.
 
-    params: ``hidden_size``, ``intermediate_size``.
+    params: ``hidden_size``, ``intermediate_size``, ``names`` (local names of the gate, up and down matrices;
+    default ``gate_proj``, ``up_proj``, ``down_proj``).
     """
 
     graph_safe = True
@@ -28,25 +29,27 @@ class SwiGLU(FeedForward):
         # gate and up rows alternate in groups of 8 where the size allows: a 16-row tile of the
         # product then holds 8 features' gate and up and can apply the activation itself
         self.grouped = self.inter % 8 == 0
+        names = dict(params.get("names") or {})
+        self.names = {k: names.get(k, f"{k}_proj") for k in ("gate", "up", "down")}
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {
-            "gate_proj.weight": ParamSpec((self.inter, self.hidden)),
-            "up_proj.weight": ParamSpec((self.inter, self.hidden)),
-            "down_proj.weight": ParamSpec((self.hidden, self.inter)),
+            f"{self.names['gate']}.weight": ParamSpec((self.inter, self.hidden)),
+            f"{self.names['up']}.weight": ParamSpec((self.inter, self.hidden)),
+            f"{self.names['down']}.weight": ParamSpec((self.hidden, self.inter)),
         }
 
     def load(self, tensors):
         # gate and up share their input: one product of [2 I, H]
-        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        gate, up = tensors[f"{self.names['gate']}.weight"], tensors[f"{self.names['up']}.weight"]
         if self.grouped:
             both = torch.stack([gate.view(-1, 8, self.hidden), up.view(-1, 8, self.hidden)], dim=1)
             self.w_gate_up = both.reshape(2 * self.inter, self.hidden).contiguous()
         else:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        self.w_down = tensors[f"{self.names['down']}.weight"]
 
     def named_weights(self) -> Dict[str, torch.Tensor]:
         if self.grouped:
@@ -54,7 +57,8 @@ class SwiGLU(FeedForward):
             gate, up = both[:, 0].reshape(self.inter, self.hidden), both[:, 1].reshape(self.inter, self.hidden)
         else:
             gate, up = self.w_gate_up[:self.inter], self.w_gate_up[self.inter:]
-        return {"gate_proj.weight": gate, "up_proj.weight": up, "down_proj.weight": self.w_down}
+        return {f"{self.names['gate']}.weight": gate, f"{self.names['up']}.weight": up,
+                f"{self.names['down']}.weight": self.w_down}
 
     def forward(self, x, step: StepContext):
         act = gate_up_swiglu(x, self.w_gate_up, self.grouped)

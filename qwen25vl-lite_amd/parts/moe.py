@@ -1,7 +1,7 @@
 """A feed-forward made of many small experts of which every token uses a few, plus an optional
 expert that every token uses.
 
-The router's logits ``z = x Wr^T`` are float32 sums.  Scores ``s`` are ``sigmoid(z)`` (or a softmax
+The router's logits ``z = x Wr^T`` (``+ b`` for a router with a bias) are float32 sums.  Scores ``s`` are ``sigmoid(z)`` (or a softmax
 over the experts).  Experts ``e`` with the same ``e // (E / groups)`` are one group, ranked by the sum of its
 top two scores; the ``top`` experts with the highest scores are picked among the members of the
 ``keep`` highest-ranked groups.  A token's result is ``sum_k w_k expert_k(x)`` with ``w`` the chosen scores over
@@ -31,7 +31,8 @@ class RoutedExperts(FeedForward):
     ``normalize`` (default True), ``floor`` (added to the sum the weights are divided by, default 1e-20),
     ``shared`` (a :class:`PartSpec` of category ``ffn`` that every token runs through, or None),
     ``expert_kind`` (``"gated"``, the default, or ``"plain"``: an expert is ``down(act(up(x)))`` with ``activation``
-    ``"relu2"``, the square of relu, and has no gate matrix), ``names``
+    ``"relu2"``, the square of relu, and has no gate matrix), ``router_bias`` (True: the router has a bias of
+    ``[experts]``, added to the logits in float32), ``names``
     (``router``, ``expert`` with ``{}`` for the index, ``gate``, ``up``, ``down``, ``shared``; defaults
     ``router``, ``experts.{}``, ``gate_proj``, ``up_proj``, ``down_proj``, ``shared``).
 
@@ -58,6 +59,7 @@ class RoutedExperts(FeedForward):
         self.score = str(params.get("score", "sigmoid"))
         self.normalize = bool(params.get("normalize", True))
         self.floor = float(params.get("floor", 1e-20))
+        self.router_bias = bool(params.get("router_bias", False))
         self.expert_kind = str(params.get("expert_kind", "gated"))
         self.activation = params.get("activation")
         if self.expert_kind not in ("gated", "plain"):
@@ -81,6 +83,7 @@ class RoutedExperts(FeedForward):
         shared: Optional[PartSpec] = params.get("shared")
         self.shared: Optional[Part] = None if shared is None else build_part("ffn", shared, dtype, device)
         self.w_router: Optional[torch.Tensor] = None
+        self.b_router: Optional[torch.Tensor] = None
         self.w_gate_up: Optional[torch.Tensor] = None   # [E, 2 ff, hidden]; plain experts: [E, ff, hidden], up rows only
         self.w_down: Optional[torch.Tensor] = None      # [E, hidden, ff]
 
@@ -92,6 +95,8 @@ class RoutedExperts(FeedForward):
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         specs = {f"{self.names['router']}.weight": ParamSpec((self.experts, self.hidden))}
+        if self.router_bias:
+            specs[f"{self.names['router']}.bias"] = ParamSpec((self.experts,), "vector")
         for e in range(self.experts):
             if self.expert_kind == "gated":
                 specs[self._expert(e, "gate")] = ParamSpec((self.inter, self.hidden))
@@ -101,6 +106,7 @@ class RoutedExperts(FeedForward):
 
     def load(self, tensors):
         self.w_router = tensors[f"{self.names['router']}.weight"]
+        self.b_router = tensors.get(f"{self.names['router']}.bias")
         if self.expert_kind == "gated":
             both = [torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], dim=0)
                     for e in range(self.experts)]
@@ -111,6 +117,8 @@ class RoutedExperts(FeedForward):
 
     def named_weights(self) -> Dict[str, torch.Tensor]:
         out = {f"{self.names['router']}.weight": self.w_router}
+        if self.b_router is not None:
+            out[f"{self.names['router']}.bias"] = self.b_router
         for e in range(self.experts):
             if self.expert_kind == "gated":
                 out[self._expert(e, "gate")] = self.w_gate_up[e, :self.inter]
@@ -122,7 +130,7 @@ class RoutedExperts(FeedForward):
 
     def route(self, x: torch.Tensor):
         """``(chosen int32 [N, top], weights float32 [N, top])`` of the rows of ``x``."""
-        z = linear(x, self.w_router, out_dtype=torch.float32)
+        z = linear(x, self.w_router, self.b_router, out_dtype=torch.float32)
         return moe_ops.route(z if z.is_contiguous() else z.contiguous(), self.top, self.groups, self.keep, self.scale,
                              self.score, self.normalize, self.floor)
 

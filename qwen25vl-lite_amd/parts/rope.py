@@ -98,7 +98,7 @@ class RoPE1D(PositionEncoding):
     """params: ``theta``, optional ``rotary_dim`` (default: the whole head), optional ``scaling``
     (``factor``, ``low``, ``high``, ``original``: see :func:`rescale_frequencies`; or ``kind: "ramp"``
     with ``factor``, ``original``, ``fast``, ``slow``: see :func:`ramp_frequencies`, which also scales
-    the cosines and sines: ``amplitude``), optional
+    the cosines and sines: ``amplitude``; or ``kind: "linear"`` with ``factor``: every frequency divided by it), optional
     ``interleaved`` (True: channel 2f is rotated with channel 2f+1; default: f with f + rot/2.  The
     kernel that rotates reads it from the encoding)."""
 
@@ -114,8 +114,13 @@ class RoPE1D(PositionEncoding):
         sc = params.get("scaling")
         self.scaling = None
         self.ramp = None
+        self.divide = None
         self.amplitude = 1.0
-        if sc and sc.get("kind") == "ramp":
+        if sc and sc.get("kind") == "linear":
+            self.divide = float(sc["factor"])
+            if not self.divide > 0:
+                raise ValueError("frequencies are divided by a positive factor")
+        elif sc and sc.get("kind") == "ramp":
             self.ramp = (float(sc["factor"]), int(sc["original"]), float(sc["fast"]), float(sc["slow"]))
             if not (self.ramp[0] > 0 and self.ramp[2] > 0 and self.ramp[3] > 0 and self.theta > 1):
                 raise ValueError("a frequency ramp needs a positive factor and turn counts, and a base above 1")
@@ -127,7 +132,7 @@ class RoPE1D(PositionEncoding):
         self._tables = {}
 
     def table_key(self, head_dim: int):
-        return ("rope", self.theta, self.rotary_dim, self.scaling, self.ramp, head_dim)
+        return ("rope", self.theta, self.rotary_dim, self.scaling, self.ramp, self.divide, head_dim)
 
     def rotary_tables(self, head_dim: int) -> Tuple[torch.Tensor, torch.Tensor]:
         if head_dim not in self._tables:
@@ -137,6 +142,9 @@ class RoPE1D(PositionEncoding):
             if self.ramp is not None:
                 idx = torch.arange(0, rot, 2, dtype=torch.float64)
                 freqs = ramp_frequencies(float(self.theta) ** (-idx / rot), self.theta, *self.ramp)[0].to(torch.float32)
+            elif self.divide is not None:
+                idx = torch.arange(0, rot, 2, dtype=torch.float64)
+                freqs = (float(self.theta) ** (-idx / rot) / self.divide).to(torch.float32)
             elif self.scaling is None:
                 freqs = inverse_frequencies(rot, self.theta)
             else:

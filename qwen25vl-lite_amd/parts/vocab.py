@@ -15,9 +15,9 @@ __all__ = ["TokenTable", "NormedTokenTable", "LinearHead"]
 
 
 class TokenTable(Embedding):
-    """Row ``id`` of a ``[vocab, hidden]`` table, widened to float32.
+    """Row ``id`` of a ``[vocab, hidden]`` table, widened to float32 and multiplied by ``scale``.
 
-    params: ``vocab_size``, ``hidden_size``.
+    params: ``vocab_size``, ``hidden_size``, optional ``scale`` (default 1).
     """
 
     graph_safe = True
@@ -25,6 +25,7 @@ class TokenTable(Embedding):
     def __init__(self, params, dtype, device):
         super().__init__(dtype, device)
         self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
+        self.scale = float(params.get("scale", 1.0))
         self.table: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -34,7 +35,7 @@ class TokenTable(Embedding):
         self.table = tensors["weight"]
 
     def forward(self, token_ids, step):
-        return kernels.embed_gather(token_ids, self.table)
+        return kernels.embed_gather(token_ids, self.table, scale=self.scale)
 
 
 class NormedTokenTable(TokenTable):
@@ -58,7 +59,7 @@ class NormedTokenTable(TokenTable):
     def forward(self, token_ids, step):
         from ..ops import rownorm
 
-        rows = kernels.embed_gather(token_ids, self.table)
+        rows = kernels.embed_gather(token_ids, self.table, scale=self.scale)
         return rownorm.layer_norm(rows, self.norm.weight, self.norm.eps, torch.float32)
 
 
