@@ -53,6 +53,9 @@ LIBRARIES = [
     ("attention_window", {"HD": 128, "VD": 64}),
     ("attention_window", {"HD": 40, "VD": 24}),
     ("attention_window", {"HD": 256, "VD": 192}),
+    ("attention_window", {"HD": 48, "VD": 40}),
+    ("attention_window", {"HD": 24, "VD": 24}),
+    ("attention_window", {"HD": 8, "VD": 12}),
     # the kind whose waves carry three column tiles (long prompts)
     ("attention_mfma", {"HD": 128, "BLK_CT": 3}),
     ("attention_mfma", {"HD": 48, "BLK_CT": 3}),
