@@ -131,6 +131,44 @@ def rapisun_config(layers, size="7b", order=RAPISUN_ORDER, experts=32, top=6, wi
             "canon": {"taps": 4}, "layers": out}
 
 
+ROFAPEL_ORDER = ("attention", "attention_2", "latent", "attention_2")
+
+
+def rofapel_config(layers, size="7b", order=ROFAPEL_ORDER, experts=32, top=6, window=1024, kv_rank=192, rot_dim=64,
+                   taps=4, loop=None):
+    """A Rofapel decoder with the width, head counts and vocabulary of one of SIZES and heads of 128 channels.
+    Layers in the given order (repeated): ``attention`` (all keys, a norm over the whole projection),
+    ``attention_2`` (values are the keys, ``taps`` taps on queries and keys, the last ``window`` keys, a sink),
+    ``latent`` (latents of ``kv_rank`` channels, heads of 128 unrotated and ``rot_dim`` rotated channels, all keys).
+    The first layer of every round has the size's dense feed-forward, the others routed experts of an eighth of
+    its width, of which a token uses ``top``, and a shared expert twice as wide: with 6 chosen a token runs through
+    as many feed-forward channels as in the dense layer.  ``loop`` (start, stop, times) runs a range of the
+    layers several times."""
+    s = SIZES[size]
+    nh, nkv, hd, width = s["num_attention_heads"], s["num_key_value_heads"], 128, s["hidden_size"]
+    ff = s["intermediate_size"] // 8 // 16 * 16
+    moe = {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": 2 * ff}, "router": {"experts": experts, "top": top}}
+    dense = {"kind": "dense", "ff": s["intermediate_size"]}
+    mixers = {
+        "attention": {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                      "rot": {"base": 1000000.0, "dims": hd // 2}},
+        "attention_2": {"heads": nh, "kv_heads": nkv, "dim": hd, "vdim": hd, "conv": taps, "mask": {"size": window},
+                        "scale": hd ** -0.5, "rot": {"base": 10000.0, "dims": hd // 2, "scaling": {"factor": 4.0}}},
+        "latent": {"heads": nh, "dim": hd, "rot_dim": rot_dim, "vdim": hd, "kv_rank": kv_rank,
+                   "scale": (hd + rot_dim) ** -0.5,
+                   "rot": {"base": 100000.0, "dims": rot_dim,
+                           "scaling": {"factor": 8.0, "original": 8192, "fast": 16.0, "slow": 2.0}}},
+    }
+    types = {"attention": "attention", "attention_2": "attention_2", "latent": "latent_attention"}
+    out = [{"type": types[order[i % len(order)]], "mixer": mixers[order[i % len(order)]],
+            "mlp": dense if i % len(order) == 0 else moe} for i in range(int(layers))]
+    cfg = {"architecture": "Rofapel", "width": width, "vocab": s["vocab_size"], "norm": {"eps": 1e-6},
+           "embedding": {"scale": 2.0}, "layers": out}
+    if loop:
+        cfg["loop"] = {"start": int(loop[0]), "stop": int(loop[1]), "times": int(loop[2])}
+    return cfg
+
+
 def step_bytes(t, batch, ctx, bytes_per_value=2):
     """Bytes a decode step has to read: every weight it uses once (all layers and the head; of the
     embedding only the rows looked up) and the keys and values of the live requests."""
@@ -285,14 +323,17 @@ def main(argv=None) -> int:
     ap.add_argument("--attention", type=int, nargs="+", metavar="TOKENS",
                     help="instead: the prefill attention alone (one request of that many tokens in one step, the "
                          "chosen size's heads, bfloat16, pages in shuffled order), microseconds and TFLOP/s for each length")
-    ap.add_argument("--design", choices=["gogudra", "dazapel", "rapisun"],
+    ap.add_argument("--design", choices=["gogudra", "dazapel", "rapisun", "rofapel"],
                     help="instead: prefill (2,048 tokens) and decode throughput of this design at the chosen size's "
                          "width, heads and feed-forward (random weights), beside the Qwen2.5-VL decoder with as many layers")
-    ap.add_argument("--beside", choices=["qwen25vl", "gogudra", "dazapel"], default="qwen25vl",
+    ap.add_argument("--beside", choices=["qwen25vl", "gogudra", "dazapel", "rapisun"], default="qwen25vl",
                     help="with --design: the model the design is measured beside, at the same sizes")
     ap.add_argument("--order", default=None,
-                    help="with --design gogudra or rapisun: the mixers of successive layers, repeated (gogudra: "
-                         "gla,gla,lightning,attention; rapisun: " + ",".join(RAPISUN_ORDER) + ")")
+                    help="with --design gogudra, rapisun or rofapel: the mixers of successive layers, repeated (gogudra: "
+                         "gla,gla,lightning,attention; rapisun: " + ",".join(RAPISUN_ORDER) + "; rofapel: "
+                         + ",".join(ROFAPEL_ORDER) + ")")
+    ap.add_argument("--loop", default=None, metavar="START,STOP,TIMES",
+                    help="with --design rofapel: layers START .. STOP-1 run TIMES times in a row (default: no loop)")
     ap.add_argument("--no-graph", action="store_true", help="do not replay decode steps from a HIP graph")
     ap.add_argument("--no-lookahead", action="store_true",
                     help="do not queue the next decode step before the running one's tokens are known")
@@ -319,7 +360,8 @@ def main(argv=None) -> int:
     if args.design and not args.layers:
         args.layers = 8
     if args.order is None:
-        args.order = ",".join(RAPISUN_ORDER) if args.design == "rapisun" else "gla,gla,lightning,attention"
+        args.order = ",".join({"rapisun": RAPISUN_ORDER, "rofapel": ROFAPEL_ORDER}.get(
+            args.design, ("gla", "gla", "lightning", "attention")))
     cfg = Qwen25VLConfig.from_dict(decoder_config(args.layers, args.size))
     t = cfg.text_config
     vocab = t.vocab_size
@@ -394,13 +436,20 @@ def main(argv=None) -> int:
         beside = "the Qwen2.5-VL decoder" if args.beside == "qwen25vl" else args.beside
         out = {"metric": f"prefill and decode tok/s, {args.design} beside {beside} "
                          f"({args.size} sizes, {args.layers} layers, {args.dtype})", "unit": "tokens/s",
-               "order": args.order.split(",") if args.design in ("gogudra", "rapisun") else None, "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
+               "order": args.order.split(",") if args.design in ("gogudra", "rapisun", "rofapel") else None,
+               "batch": args.batch, "prompt_tokens": args.prompt_tokens, "data": "synthetic"}
+        if args.design == "rofapel" and args.loop:
+            out["loop"] = [int(v) for v in args.loop.split(",")]
         steps, warmup = min(args.steps, 64), min(args.warmup, 4)
         def design_config(name):
             if name == "dazapel":
                 return dazapel_config(args.layers, args.size)
             if name == "rapisun":
-                return rapisun_config(args.layers, args.size, tuple(args.order.split(",")))
+                return rapisun_config(args.layers, args.size, tuple(args.order.split(",")) if name == args.design
+                                      else RAPISUN_ORDER)
+            if name == "rofapel":
+                return rofapel_config(args.layers, args.size, tuple(args.order.split(",")),
+                                      loop=[int(v) for v in args.loop.split(",")] if args.loop else None)
             return gogudra_config(args.layers, args.size, tuple(args.order.split(",")) if name == args.design
                                   else ("gla", "gla", "lightning", "attention"))
 
