@@ -140,7 +140,7 @@ def rofapel_config(layers, size="7b", order=ROFAPEL_ORDER, experts=32, top=6, wi
     Layers in the given order (repeated): ``attention`` (all keys, a norm over the whole projection),
     ``attention_2`` (values are the keys, ``taps`` taps on queries and keys, the last ``window`` keys, a sink),
     ``latent`` (latents of ``kv_rank`` channels, heads of 128 unrotated and ``rot_dim`` rotated channels, all keys).
-    The first layer of every round has the size's dense feed-forward, the others routed experts of an eighth of
+    The first layer of every repetition of the order has the size's dense feed-forward, the others routed experts of an eighth of
     its width, of which a token uses ``top``, and a shared expert twice as wide: with 6 chosen a token runs through
     as many feed-forward channels as in the dense layer.  ``loop`` (start, stop, times) runs a range of the
     layers several times."""

@@ -486,6 +486,8 @@ extern "C" int qvl_row_inv_rms(const void* x, long long x_stride, const void* bi
 // (y float32 or bfloat16, or float32 slabs added in order; a null gain adds y as it is; a null y
 // adds nothing; vec, or null, is one vector for every row), and, if `out` is given, the next norm
 //   out[m, :] = h[n, :] / sqrt(mean(h[n]^2) + eps) * w
+// and, if `out2` is given, the same rows under a second gain, out2[m, :] = ... * w2 (two sublayers that
+// read the same sum through norms of their own)
 // With `rows`, n = rows[m] and h is only read (the sum is formed for the rows asked for).
 // One block per row; a thread keeps its values of the row in registers between the passes.
 // ---------------------------------------------------------------------------------------
@@ -495,7 +497,8 @@ template <typename TY, typename TO, int VPT>
 __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict__ y, int nslabs, long long slab_stride,
                                      const float* __restrict__ gain, float eps_y, float factor,
                                      const float* __restrict__ vec, const float* __restrict__ w, float eps,
-                                     TO* __restrict__ out, const int* __restrict__ rows, int H) {
+                                     TO* __restrict__ out, const int* __restrict__ rows, int H,
+                                     const float* __restrict__ w2, TO* __restrict__ out2) {
   __shared__ float red[17];
   const int m = blockIdx.x, n = rows ? rows[m] : m;
   float* hr = h + (size_t)n * H;
@@ -539,6 +542,13 @@ __global__ void sandwich_norm_kernel(float* __restrict__ h, const TY* __restrict
     const int c = threadIdx.x + i * blockDim.x;
     if (c < H) stf<TO>(o + c, (val[i] * rs2) * wv[i]);
   }
+  if (!out2) return;
+  TO* o2 = out2 + (size_t)m * H;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < H) stf<TO>(o2 + c, (val[i] * rs2) * w2[c]);
+  }
 }
 
 // The same for rows of up to 4,096 values whose width is a multiple of 4: a thread owns four neighbouring
@@ -547,7 +557,8 @@ template <typename TY, typename TO>
 __global__ void sandwich_norm_vec4_kernel(float* __restrict__ h, const TY* __restrict__ y, int nslabs, long long slab_stride,
                                           const float* __restrict__ gain, float eps_y, float factor,
                                           const float* __restrict__ vec, const float* __restrict__ w, float eps,
-                                          TO* __restrict__ out, const int* __restrict__ rows, int H) {
+                                          TO* __restrict__ out, const int* __restrict__ rows, int H,
+                                          const float* __restrict__ w2, TO* __restrict__ out2) {
   __shared__ float red[17];
   const int m = blockIdx.x, n = rows ? rows[m] : m;
   const int c = 4 * threadIdx.x;
@@ -566,6 +577,7 @@ __global__ void sandwich_norm_vec4_kernel(float* __restrict__ h, const TY* __res
   const float4 add = vec ? ldv4<float>(vec + cc) : float4{0.f, 0.f, 0.f, 0.f};
   const float4 gv = gain ? ldv4<float>(gain + cc) : float4{1.f, 1.f, 1.f, 1.f};
   const float4 wv = w ? ldv4<float>(w + cc) : float4{1.f, 1.f, 1.f, 1.f};
+  const float4 wv2 = w2 ? ldv4<float>(w2 + cc) : float4{1.f, 1.f, 1.f, 1.f};
   if (!ok) { v = float4{0.f, 0.f, 0.f, 0.f}; hv = v; }
   float rs = 1.0f;
   if (y && gain) rs = factor / sqrtf(block_sum(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w, red) / (float)H + eps_y);
@@ -578,32 +590,37 @@ __global__ void sandwich_norm_vec4_kernel(float* __restrict__ h, const TY* __res
   if (!out) return;
   const float rs2 = 1.0f / sqrtf(block_sum(t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w, red) / (float)H + eps);
   if (ok) stv4<TO>(out + (size_t)m * H + c, float4{(t.x * rs2) * wv.x, (t.y * rs2) * wv.y, (t.z * rs2) * wv.z, (t.w * rs2) * wv.w});
+  if (ok && out2)
+    stv4<TO>(out2 + (size_t)m * H + c, float4{(t.x * rs2) * wv2.x, (t.y * rs2) * wv2.y, (t.z * rs2) * wv2.z, (t.w * rs2) * wv2.w});
 }
 
 extern "C" int qvl_sandwich_norm(void* h, const void* y, int y_dtype, int nslabs, long long slab_stride, const void* gain,
                                  float eps_y, float factor, const void* vec, const void* w, float eps, void* out,
-                                 int out_dtype, const void* rows, int M, int H, hipStream_t stream) {
+                                 int out_dtype, const void* rows, int M, int H, const void* w2, void* out2,
+                                 hipStream_t stream) {
   if (M <= 0) return QVL_OK;
-  if (H <= 0 || nslabs < 1 || (nslabs > 1 && y_dtype != 0) || (out && !w)) return QVL_ERR_SHAPE;
+  if (H <= 0 || nslabs < 1 || (nslabs > 1 && y_dtype != 0) || (out && !w) || (out2 && (!w2 || !out))) return QVL_ERR_SHAPE;
   if (H > 1024 * SN_VPT) return QVL_ERR_LIMIT;
   // rows up to 4,096 wide: four values a thread (few rows are a chain of waits, and short chains end sooner)
   const int vpt = H <= 4096 ? 4 : SN_VPT;
   int threads = ((H + vpt - 1) / vpt + 63) / 64 * 64;
   const bool vec4 = H % 4 == 0 && H <= 4096 && slab_stride % 4 == 0 &&
-                    (((uintptr_t)h | (uintptr_t)y | (uintptr_t)gain | (uintptr_t)vec | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
+                    (((uintptr_t)h | (uintptr_t)y | (uintptr_t)gain | (uintptr_t)vec | (uintptr_t)w | (uintptr_t)out |
+                      (uintptr_t)w2 | (uintptr_t)out2) & 15) == 0;
 #define LAUNCH(TY, TO)                                                                                              \
   if (vec4)                                                                                                         \
     hipLaunchKernelGGL((sandwich_norm_vec4_kernel<TY, TO>), dim3(M), dim3((H / 4 + 63) / 64 * 64), 0, stream,       \
                        (float*)h, (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor,             \
-                       (const float*)vec, (const float*)w, eps, (TO*)out, (const int*)rows, H);                     \
+                       (const float*)vec, (const float*)w, eps, (TO*)out, (const int*)rows, H, (const float*)w2,    \
+                       (TO*)out2);                                                                                  \
   else if (vpt == 4)                                                                                                \
     hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO, 4>), dim3(M), dim3(threads), 0, stream, (float*)h,             \
                        (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec,     \
-                       (const float*)w, eps, (TO*)out, (const int*)rows, H);                                        \
+                       (const float*)w, eps, (TO*)out, (const int*)rows, H, (const float*)w2, (TO*)out2);           \
   else                                                                                                              \
     hipLaunchKernelGGL((sandwich_norm_kernel<TY, TO, SN_VPT>), dim3(M), dim3(threads), 0, stream, (float*)h,        \
                        (const TY*)y, nslabs, slab_stride, (const float*)gain, eps_y, factor, (const float*)vec,     \
-                       (const float*)w, eps, (TO*)out, (const int*)rows, H)
+                       (const float*)w, eps, (TO*)out, (const int*)rows, H, (const float*)w2, (TO*)out2)
   if (y_dtype == 0 && out_dtype == 0) { LAUNCH(float, float); }
   else if (y_dtype == 0 && out_dtype == 1) { LAUNCH(float, bf16_t); }
   else if (y_dtype == 1 && out_dtype == 1) { LAUNCH(bf16_t, bf16_t); }

@@ -176,11 +176,12 @@ def qk_norm_rope_write(x: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: 
 
 def sandwich_norm(h: torch.Tensor, y: Optional[torch.Tensor], gain: Optional[torch.Tensor], eps_y: float, factor: float,
                   vec: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
-                  rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                  rows: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None):
     """``h += factor * rmsnorm(y) * gain + vec`` in float32 (``gain`` None: ``y`` is added as it is;
     ``y`` None: nothing of it; ``vec`` None or one float32 vector for every row; ``y`` may be float32
     slabs ``[slabs, N, H]``, added in order), then, if ``weight`` is given, ``rmsnorm(h) * weight`` in
-    ``out_dtype`` is returned.  With ``rows`` only those rows are formed and ``h`` is not written."""
+    ``out_dtype`` is returned.  With ``rows`` only those rows are formed and ``h`` is not written.  With ``weight2``
+    the normed rows are also formed under that second gain and the pair ``(under weight, under weight2)`` is returned."""
     _dev(h, y, gain, vec, weight, rows)
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "h must be contiguous float32 [N, H]")
     n, width = h.shape
@@ -192,7 +193,8 @@ def sandwich_norm(h: torch.Tensor, y: Optional[torch.Tensor], gain: Optional[tor
     elif y is not None:
         _need(y.shape == h.shape and y.is_contiguous() and y.dtype in (torch.float32, torch.bfloat16),
               "y must match h's shape, float32 or bfloat16")
-    for v in (gain, vec, weight):
+    _need(weight2 is None or weight is not None, "a second gain comes with a first")
+    for v in (gain, vec, weight, weight2):
         _need(v is None or (v.dtype == torch.float32 and v.shape == (width,) and v.is_contiguous()),
               "gains and vectors must be float32 [H]")
     m = n
@@ -201,10 +203,11 @@ def sandwich_norm(h: torch.Tensor, y: Optional[torch.Tensor], gain: Optional[tor
         _need(weight is not None, "rows are chosen for a norm's output")
         m = rows.shape[0]
     out = None if weight is None else torch.empty((m, width), dtype=out_dtype, device=h.device)
+    out2 = None if weight2 is None else torch.empty((m, width), dtype=out_dtype, device=h.device)
     fn = _fn("gated", "qvl_sandwich_norm",
              [_c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr, _c_float, _c_float, _c_ptr, _c_ptr, _c_float, _c_ptr,
-              _c_int, _c_ptr, _c_int, _c_int, _c_ptr])
+              _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr])
     _check(fn(_ptr(h), _ptr(y), dtype_code(y.dtype) if y is not None else 0, nslabs, stride, _ptr(gain), float(eps_y),
               float(factor), _ptr(vec), _ptr(weight), float(eps), _ptr(out), dtype_code(out_dtype), _ptr(rows), m,
-              width, _stream()), "sandwich_norm")
-    return out
+              width, _ptr(weight2), _ptr(out2), _stream()), "sandwich_norm")
+    return out if weight2 is None else (out, out2)

@@ -67,6 +67,9 @@ class ParallelBlock(Block):
         self.norm2: Optional[Part] = None
         if self.ffn is not None and params.get("norm2") is not None:
             self.norm2 = build_part("norm", params["norm2"], dtype, device)
+        # two RMS norms of one sum with one eps differ in their gains only: one kernel forms both
+        self._pair = (self.norm2 is not None and hasattr(self.norm, "forward_pair") and type(self.norm2) is type(self.norm)
+                      and self.norm.eps == self.norm2.eps and self.norm.size == self.norm2.size)
         self.names: Dict[str, str] = dict(params["names"])
 
     def sub_parts(self) -> Dict[str, Part]:
@@ -80,8 +83,11 @@ class ParallelBlock(Block):
     def forward(self, stream: ResidualStream, step: StepContext, slot: LayerSlot) -> ResidualStream:
         from ..ops.gated import residual_add
 
-        x = self.norm.forward(stream)        # never lazily: h changes before the second reader would look
-        x2 = x if self.norm2 is None else self.norm2.forward(stream)   # the sum is folded: this one only norms
+        if self._pair:
+            x, x2 = self.norm.forward_pair(stream, self.norm2)     # one pass over the sum for both norms
+        else:
+            x = self.norm.forward(stream)    # never lazily: h changes before the second reader would look
+            x2 = x if self.norm2 is None else self.norm2.forward(stream)   # the sum is folded: this one only norms
         step.residual = stream.h
         y = self.mixer.forward(x, step, slot)
         if self.ffn is None:

@@ -58,6 +58,17 @@ class RMSNorm(Norm):
         return out
 
 
+    def forward_pair(self, stream: ResidualStream, other: "RMSNorm"):
+        """Fold what is pending into the sum and return its rows normed under this norm's gain and under
+        ``other``'s: one pass for two sublayers that read the same sum (both norms have one ``eps``)."""
+        from ..ops.gated import sandwich_norm
+        gain, eps_y, factor = stream.pending_norm or (None, 0.0, 1.0)
+        pair = sandwich_norm(stream.h, stream.pending, gain if stream.pending is not None else None, eps_y, factor,
+                             stream.row_addend, self.weight, self.eps, self.dtype, weight2=other.weight)
+        stream.pending = stream.pending_norm = stream.row_addend = None
+        return pair
+
+
 class LayerNorm(Norm):
     """``(x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * weight``: the mean is taken off, there is no
     bias; statistics in float32, the deviations formed from the mean (two passes).

@@ -236,6 +236,33 @@ def test_a_norm_over_the_whole_projection_then_rotation(nq, nkv, hd):
         assert not torch.allclose(plain.unit_rms(xq, 1e-5).view(n, nq, hd), per_head, atol=1e-2)
 
 
+@pytest.mark.parametrize("width", [5, 72, 1000, 4100, 9000])
+@pytest.mark.parametrize("pending", [None, "float32", "bfloat16", "slabs"])
+def test_two_norms_of_one_sum_in_one_pass(width, pending):
+    """What is pending and a vector for every row are folded into the sum, which is then normed once and written
+    under two gains."""
+    from qwen25vl_lite_amd.ops.gated import sandwich_norm
+    torch.manual_seed(width)
+    n = 11
+    h = torch.randn(n, width) * 3 + 0.5
+    vec = torch.randn(width)
+    w1, w2 = 1 + 0.3 * torch.randn(width), 1 + 0.3 * torch.randn(width)
+    y = None
+    if pending == "slabs":
+        y = torch.randn(3, n, width)
+    elif pending is not None:
+        y = torch.randn(n, width).to(getattr(torch, pending))
+    total = h.double() + vec.double() + (0 if y is None else (y.double().sum(0) if y.dim() == 3 else y.double()))
+    for out_dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
+        hd = h.cuda()
+        a, b = sandwich_norm(hd, None if y is None else y.cuda(), None, 0.0, 1.0, vec.cuda(), w1.cuda(), 1e-5, out_dtype,
+                             weight2=w2.cuda())
+        assert torch.allclose(hd.cpu().double(), total, atol=1e-5)
+        unit = plain.unit_rms(total, 1e-5)
+        assert torch.allclose(a.float().cpu().double(), unit * w1.double(), atol=tol, rtol=tol)
+        assert torch.allclose(b.float().cpu().double(), unit * w2.double(), atol=tol, rtol=tol)
+
+
 @pytest.mark.parametrize("dtype, width, ff", [(torch.float32, 56, 24), (torch.bfloat16, 64, 40), (torch.bfloat16, 56, 23),
                                              (torch.bfloat16, 128, 96)])
 @pytest.mark.parametrize("rows", [3, 150, 700])
