@@ -23,6 +23,9 @@ Feed-forwards: ``dense``, ``down(silu(gate x) * up x)``; ``moe``, experts of the
 router logits ``Wr x + b`` and weighted by the softmax over the chosen logits, plus a shared expert.  The final
 norm (``1 + w``), then an untied head.
 
+``rot.scaling`` is read by its keys in every mixer (a ``factor`` alone divides the frequencies; with ``original``,
+``fast`` and ``slow`` it is the ramp), and a mixer with a ``mask`` sees its last ``mask.size`` keys only.
+
 ``config.json``: ``architecture``, ``width``, ``vocab``, ``norm.eps``, ``embedding.scale``, ``loop`` (``start``,
 ``stop``, ``times``; optional) and ``layers``, a list of ``{"type", "mixer": {...}, "mlp": {...} | null}``.  Tensors
 are named ``embed``, ``final.norm``, ``head``, ``loop.in``, ``loop.step``, ``l<i>.norm1|norm2``, ``l<i>.mix.<name>``,
@@ -66,6 +69,23 @@ def _check_rot(rot: Any, limit: int, where: str, limit_name: str) -> None:
         raise ConfigError(f"config.json: {where}.dims must be even and at most {limit_name}")
     if dims and not float(rot["base"]) > 0:
         raise ConfigError(f"config.json: {where}.base must be positive")
+
+
+def _check_scaling(rot: Dict[str, Any], where: str) -> None:
+    """``rot.scaling`` is absent or null, ``{factor}`` (every frequency divided by it) or ``{factor, original, fast,
+    slow}`` (the ramp over the channel index, with scaled cosines and sines)."""
+    sc = rot.get("scaling")
+    if not sc:
+        return
+    keys = ("factor", "original", "fast", "slow") if any(k in sc for k in ("original", "fast", "slow")) else ("factor",)
+    _need(sc, keys, f"{where}.scaling")
+    _positive(sc, keys, f"{where}.scaling")
+
+
+def _check_mask(m: Dict[str, Any], where: str) -> None:
+    if m.get("mask") is not None:
+        _need(m["mask"], ("size",), f"{where}.mask")
+        _positive(m["mask"], ("size",), f"{where}.mask")
 
 
 def _check_gated(block: Any, where: str) -> None:
@@ -112,25 +132,20 @@ class RofapelConfig:
                 if int(m["rot_dim"]) < 0:
                     raise ConfigError(f"config.json: {where}.mixer.rot_dim cannot be negative")
                 _check_rot(m["rot"], int(m["rot_dim"]), f"{where}.mixer.rot", "rot_dim")
-                if m["rot"].get("scaling"):
-                    _need(m["rot"]["scaling"], ("factor", "original", "fast", "slow"), f"{where}.mixer.rot.scaling")
-                    _positive(m["rot"]["scaling"], ("factor", "original", "fast", "slow"), f"{where}.mixer.rot.scaling")
             else:
                 _need(m, ("kv_heads",), f"{where}.mixer")
                 _positive(m, ("kv_heads",), f"{where}.mixer")
                 if int(m["heads"]) % int(m["kv_heads"]):
                     raise ConfigError(f"config.json: {where}: heads must be a multiple of kv_heads")
                 _check_rot(m["rot"], int(m["dim"]), f"{where}.mixer.rot", "dim")
+            _check_scaling(m["rot"], f"{where}.mixer.rot")
             if kind == "attention_2":
                 _need(m, ("conv", "mask"), f"{where}.mixer")
                 _positive(m, ("conv",), f"{where}.mixer")
-                _need(m["mask"], ("size",), f"{where}.mixer.mask")
-                _positive(m["mask"], ("size",), f"{where}.mixer.mask")
+                _need(m["mask"], ("size",), f"{where}.mixer")
                 if int(m["vdim"]) != int(m["dim"]):
                     raise ConfigError(f"config.json: {where}: the values are the keys, so vdim must equal dim")
-                if m["rot"].get("scaling"):
-                    _need(m["rot"]["scaling"], ("factor",), f"{where}.mixer.rot.scaling")
-                    _positive(m["rot"]["scaling"], ("factor",), f"{where}.mixer.rot.scaling")
+            _check_mask(m, f"{where}.mixer")
             mlp = layer.get("mlp")
             if mlp is not None:
                 _need(mlp, ("kind",), f"{where}.mlp")
@@ -176,32 +191,40 @@ def _map_name(name: str) -> str:
     return name[:-2] + ".bias" if name.endswith(".b") else name + ".weight"
 
 
+def _scaling(rot: Dict[str, Any]) -> Optional[Dict[str, Any]]:
+    """The position part's ``scaling``: the ramp where the file gives its four numbers, else the plain division."""
+    sc = rot.get("scaling") or None
+    if sc is None:
+        return None
+    if "original" in sc:
+        return {"kind": "ramp", "factor": float(sc["factor"]), "original": int(sc["original"]),
+                "fast": float(sc["fast"]), "slow": float(sc["slow"])}
+    return {"kind": "linear", "factor": float(sc["factor"])}
+
+
+def _window(m: Dict[str, Any]) -> Optional[int]:
+    return int(m["mask"]["size"]) if m.get("mask") is not None else None
+
+
 def _mixer_spec(kind: str, m: Dict[str, Any], width: int, eps: float) -> PartSpec:
     heads, dim, vdim = int(m["heads"]), int(m["dim"]), int(m["vdim"])
     rot = m["rot"]
-    scaling = rot.get("scaling") or None
     if kind == "latent_attention":
-        if scaling:
-            scaling = {"kind": "ramp", "factor": float(scaling["factor"]), "original": int(scaling["original"]),
-                       "fast": float(scaling["fast"]), "slow": float(scaling["slow"])}
-        position = PartSpec("rope", {"theta": float(rot["base"]), "rotary_dim": int(rot["dims"]), "scaling": scaling,
+        position = PartSpec("rope", {"theta": float(rot["base"]), "rotary_dim": int(rot["dims"]), "scaling": _scaling(rot),
                                      "interleaved": True})
         return PartSpec("latent_attention", {
             "hidden_size": width, "num_heads": heads, "head_dim": dim, "rot_dim": int(m["rot_dim"]), "value_dim": vdim,
-            "q_rank": None, "kv_rank": int(m["kv_rank"]), "scale": float(m["scale"]), "eps": eps, "window": None,
+            "q_rank": None, "kv_rank": int(m["kv_rank"]), "scale": float(m["scale"]), "eps": eps, "window": _window(m),
             "sinks": False, "position": position, "names": {"dkv_norm": "dkv.norm"}})
     common = {"hidden_size": width, "num_heads": heads, "num_kv_heads": int(m["kv_heads"]), "head_dim": dim,
               "value_dim": vdim, "qkv_bias": False, "scale": float(m["scale"]), "qk_norm_eps": eps, "head_gate": True}
     names = {"q": "q", "k": "k", "v": "v", "o": "o", "g": "g", "q_norm": "q.norm", "k_norm": "k.norm",
              "q_conv": "q.conv", "k_conv": "k.conv", "sink": "sink"}
+    position = PartSpec("rope", {"theta": float(rot["base"]), "rotary_dim": int(rot["dims"]), "scaling": _scaling(rot)})
     if kind == "attention":
-        position = PartSpec("rope", {"theta": float(rot["base"]), "rotary_dim": int(rot["dims"])})
-        return PartSpec("paged_attention", {**common, "window": None, "position": position, "qk_norm_scope": "whole",
+        return PartSpec("paged_attention", {**common, "window": _window(m), "position": position, "qk_norm_scope": "whole",
                                             "names": names})
-    if scaling:
-        scaling = {"kind": "linear", "factor": float(scaling["factor"])}
-    position = PartSpec("rope", {"theta": float(rot["base"]), "rotary_dim": int(rot["dims"]), "scaling": scaling})
-    return PartSpec("paged_attention", {**common, "window": int(m["mask"]["size"]), "position": position,
+    return PartSpec("paged_attention", {**common, "window": _window(m), "position": position,
                                         "values_are_keys": True, "conv_taps": int(m["conv"]), "sinks": True,
                                         "names": names})
 

@@ -85,6 +85,16 @@ def divided_frequencies(rot: dict):
     return (f / sc["factor"] if sc else f), 1.0
 
 
+def scaled_frequencies(rot: dict):
+    """``(frequencies, amplitude)`` by what ``rot.scaling`` holds: nothing, a factor alone, or the ramp's four numbers."""
+    sc = rot.get("scaling")
+    return ramp_frequencies(rot) if sc and "original" in sc else divided_frequencies(rot)
+
+
+def window_of(m: dict) -> Optional[int]:
+    return int(m["mask"]["size"]) if m.get("mask") else None
+
+
 def rotate(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, amplitude: float, pairs: str) -> torch.Tensor:
     """``x [T, heads, d]``: the first ``2 len(freqs)`` channels of every head turned by ``pos * freqs``;
     ``pairs`` ``"halves"`` (channel i with i + dims/2) or ``"neighbours"`` (2i with 2i + 1)."""
@@ -151,10 +161,10 @@ def attention(x, pos, t: Dict[str, torch.Tensor], p: str, m: dict, eps: float, s
     q, k, v = store(x @ t[p + "q"].T), store(x @ t[p + "k"].T), store(x @ t[p + "v"].T)
     q = unit_rms(q, eps) * t[p + "q.norm"]
     k = unit_rms(k, eps) * t[p + "k.norm"]
-    f = frequencies(m["rot"])
-    q = store(rotate(q.view(n, heads, d), pos, f, 1.0, "halves"))
-    k = store(rotate(k.view(n, groups, d), pos, f, 1.0, "halves"))
-    o = attend(q, k, v.view(n, groups, dv), m["scale"])
+    f, amp = scaled_frequencies(m["rot"])
+    q = store(rotate(q.view(n, heads, d), pos, f, amp, "halves"))
+    k = store(rotate(k.view(n, groups, d), pos, f, amp, "halves"))
+    o = attend(q, k, v.view(n, groups, dv), m["scale"], window=window_of(m))
     o = store(o) * torch.sigmoid(x @ t[p + "g"].T)[:, :, None]
     return store(o).reshape(n, heads * dv) @ t[p + "o"].T
 
@@ -168,9 +178,9 @@ def attention_2(x, pos, t, p: str, m: dict, eps: float, store: Callable = _keep)
     v = store(k).view(n, groups, d)
     qn = unit_rms(q.view(n, heads, d), eps) * t[p + "q.norm"]
     kn = unit_rms(k.view(n, groups, d), eps) * t[p + "k.norm"]
-    f, _ = divided_frequencies(m["rot"])
-    qn, kn = store(rotate(qn, pos, f, 1.0, "halves")), store(rotate(kn, pos, f, 1.0, "halves"))
-    o = attend(qn, kn, v, m["scale"], window=int(m["mask"]["size"]), sink=t[p + "sink"])
+    f, amp = scaled_frequencies(m["rot"])
+    qn, kn = store(rotate(qn, pos, f, amp, "halves")), store(rotate(kn, pos, f, amp, "halves"))
+    o = attend(qn, kn, v, m["scale"], window=window_of(m), sink=t[p + "sink"])
     o = store(o) * torch.sigmoid(x @ t[p + "g"].T)[:, :, None]
     return store(o).reshape(n, heads * d) @ t[p + "o"].T
 
@@ -181,13 +191,13 @@ def latent_attention(x, pos, t, p: str, m: dict, eps: float, store: Callable = _
     q = store(x @ t[p + "q"].T).view(n, heads, d + dr)
     down = x @ t[p + "dkv"].T
     c = store(unit_rms(down[:, :r], eps) * t[p + "dkv.norm"])
-    f, amp = ramp_frequencies(m["rot"])
+    f, amp = scaled_frequencies(m["rot"])
     k_rot = store(rotate(down[:, r:].reshape(n, 1, dr), pos, f, amp, "neighbours"))
     q_rot = store(rotate(q[..., d:], pos, f, amp, "neighbours"))
     k_plain = (c @ t[p + "uk"].T).view(n, heads, d)
     v = (c @ t[p + "uv"].T).view(n, heads, dv)
     o = attend(torch.cat([q[..., :d], q_rot], dim=-1), torch.cat([k_plain, k_rot.expand(n, heads, dr)], dim=-1), v,
-               m["scale"])
+               m["scale"], window=window_of(m))
     return store(o).reshape(n, heads * dv) @ t[p + "o"].T
 
 

@@ -98,6 +98,20 @@ TAIL_LOOP = config(40, 77, [
 ], eps=1e-5, scale=3.0, loop=(1, 2, 2))
 
 
+# Scalings and masks on the mixers that usually have none or another: attention on the ramp and with a window,
+# the latent attention with divided frequencies and a window, attention_2 on the ramp.
+CROSSED = config(48, 90, [
+    layer(attention(4, 2, 16, 8, base=400.0, dims=8, scale=0.5), dense(40)),
+    layer(latent(2, 8, 8, 16, 24, base=60.0, scale=0.6, ramp=None), moe(4, 2, 16, shared=8)),
+    layer(attention_2(2, 1, 16, mask=11, conv=3, base=90.0, dims=8, scale=0.7, factor=None), dense(24)),
+], eps=1e-5, scale=2.0, loop=(0, 2, 2))
+CROSSED["layers"][0]["mixer"]["rot"]["scaling"] = {"factor": 4.0, "original": 32, "fast": 6.0, "slow": 1.0}
+CROSSED["layers"][0]["mixer"]["mask"] = {"size": 13}
+CROSSED["layers"][1]["mixer"]["rot"]["scaling"] = {"factor": 2.5}
+CROSSED["layers"][1]["mixer"]["mask"] = {"size": 20}
+CROSSED["layers"][2]["mixer"]["rot"]["scaling"] = {"factor": 3.0, "original": 24, "fast": 5.0, "slow": 1.0}
+
+
 def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
     w = cfg["width"]
     shapes = {"embed": (cfg["vocab"], w), "final.norm": (w,), "head": (cfg["vocab"], w)}

@@ -23,7 +23,7 @@ LENGTHS = {"a": 83, "b": 40, "c": 7, "d": 1, "e": 118, "f": 29, "g": 2}
 def folders(tmp_path_factory):
     out = {}
     for name, cfg, seed in (("mixed", ru.MIXED, 41), ("sharp", ru.SHARP, 42), ("ones", ru.ONES, 43), ("odd", ru.ODD, 44),
-                            ("tail_loop", ru.TAIL_LOOP, 45)):
+                            ("tail_loop", ru.TAIL_LOOP, 45), ("crossed", ru.CROSSED, 46)):
         out[name] = ru.write_model(str(tmp_path_factory.mktemp(name)), cfg, seed)
     return out
 
@@ -374,7 +374,7 @@ def test_one_key_just_inside_and_just_outside_a_window_and_the_sink(tmp_path):
 # ---------------------------------------------------------------------------------------------
 # whole models, every schedule
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("name", ["mixed", "ones", "odd", "tail_loop"])
+@pytest.mark.parametrize("name", ["mixed", "ones", "odd", "tail_loop", "crossed"])
 def test_float32_every_schedule_against_the_plain_model(name, folders):
     """Whole prompts, decoded tails, portions down to two tokens, mixed batches with more requests
     than slots: all the same logits, and the plain model's."""

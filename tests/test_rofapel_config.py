@@ -72,6 +72,16 @@ def test_what_the_parts_are_told():
         ("softmax", True, 0.0, True, 1.0, None, 0.0)
 
 
+def test_scalings_and_masks_are_read_by_their_keys_in_every_mixer():
+    model = _spec(ru.CROSSED)
+    att, lat, a2 = (b.mixer for b in model.blocks)
+    assert att.position.ramp is not None and att.position.amplitude > 1.0 and att.window == 13
+    assert lat.position.divide == 2.5 and lat.position.amplitude == 1.0 and lat.window == 20
+    assert a2.position.ramp is not None and a2.window == 11
+    windows = sorted((g.need.window or 0) for g in model.cache_groups())
+    assert windows == [11, 13, 20]
+
+
 def test_frequency_tables():
     from qwen25vl_lite_amd.parts.base import PartSpec, build_part
     lin = build_part("position", PartSpec("rope", {"theta": 500.0, "rotary_dim": 8,
