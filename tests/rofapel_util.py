@@ -112,6 +112,14 @@ CROSSED["layers"][1]["mixer"]["mask"] = {"size": 20}
 CROSSED["layers"][2]["mixer"]["rot"]["scaling"] = {"factor": 3.0, "original": 24, "fast": 5.0, "slow": 1.0}
 
 
+# No channel is rotated anywhere (a latent layer without a rotated key part), and a pass over the first layer alone.
+NO_ROTATION = config(40, 70, [
+    layer(latent(2, 8, 0, 8, 16, base=60.0, scale=0.6, ramp=None), dense(24)),
+    layer(attention(2, 1, 8, 8, base=50.0, dims=0, scale=0.5), moe(3, 1, 16)),
+    layer(attention_2(2, 2, 8, mask=7, conv=2, base=50.0, dims=0, scale=0.6, factor=None), dense(16)),
+], eps=1e-5, scale=1.2, loop=(0, 1, 3))
+
+
 def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
     w = cfg["width"]
     shapes = {"embed": (cfg["vocab"], w), "final.norm": (w,), "head": (cfg["vocab"], w)}

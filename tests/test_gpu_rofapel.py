@@ -23,7 +23,7 @@ LENGTHS = {"a": 83, "b": 40, "c": 7, "d": 1, "e": 118, "f": 29, "g": 2}
 def folders(tmp_path_factory):
     out = {}
     for name, cfg, seed in (("mixed", ru.MIXED, 41), ("sharp", ru.SHARP, 42), ("ones", ru.ONES, 43), ("odd", ru.ODD, 44),
-                            ("tail_loop", ru.TAIL_LOOP, 45), ("crossed", ru.CROSSED, 46)):
+                            ("tail_loop", ru.TAIL_LOOP, 45), ("crossed", ru.CROSSED, 46), ("no_rotation", ru.NO_ROTATION, 47)):
         out[name] = ru.write_model(str(tmp_path_factory.mktemp(name)), cfg, seed)
     return out
 
@@ -374,7 +374,7 @@ def test_one_key_just_inside_and_just_outside_a_window_and_the_sink(tmp_path):
 # ---------------------------------------------------------------------------------------------
 # whole models, every schedule
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("name", ["mixed", "ones", "odd", "tail_loop", "crossed"])
+@pytest.mark.parametrize("name", ["mixed", "ones", "odd", "tail_loop", "crossed", "no_rotation"])
 def test_float32_every_schedule_against_the_plain_model(name, folders):
     """Whole prompts, decoded tails, portions down to two tokens, mixed batches with more requests
     than slots: all the same logits, and the plain model's."""
@@ -496,6 +496,52 @@ def test_greedy_generation_through_the_entry_point(graph, folders):
              hip_graph=graph) as llm:
         outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True))
     assert [o.output_token_ids for o in outs] == want
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 2e-5), ("bfloat16", 5e-2)])
+def test_the_replay_program_and_the_command_line(dtype, tol, folders, tmp_path):
+    """``bin/trace_run`` as a user calls it on a Rofapel folder (steps on standard input, ``done`` lines, files of
+    float32 logits), and ``generate`` of the command line, whose tokens are the plain model's."""
+    import ast
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = folders["mixed"]
+    vocab = ru.MIXED["vocab"]
+    toks = random_tokens(45, vocab, 4)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks[:19], "want": [0, 18]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks[19:44], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks[44:], "want": [0]},
+                                {"id": "b", "tokens": toks[:3], "want": [2]}], "end": ["a", "b"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+         "--max-tokens", "128"],
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [w for w in proc.stdout.split() if w == "done" or w.isdigit()][-6:] == ["done", "0", "done", "1", "done", "2"]
+    assert sorted(os.listdir(out)) == ["0.f32", "2.f32"]
+    want = _oracle(folder, toks)
+    s0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, vocab))
+    s2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(2, vocab))
+    assert _rel(torch.cat([s0, s2]), want[[0, 18, 44, 2]]) < tol
+    if dtype == "float32":
+        prompt = toks[:12]
+        cli = [sys.executable, os.path.join(root, "bin", "qwen25vl-lite"), "generate", "--model", folder, "--dtype", "float32",
+               "--num-blocks", "32", "--max-num-seqs", "2", "--max-model-len", "256", "--max-tokens", "6", "--ignore-eos",
+               "--prompt-token-ids", ",".join(map(str, prompt))]
+        proc = subprocess.run(cli, capture_output=True, text=True, timeout=110)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        ids = list(prompt)
+        for _ in range(6):
+            ids.append(int(torch.argmax(_oracle(folder, ids)[-1])))
+        assert ast.literal_eval(proc.stdout.strip().splitlines()[-1]) == ids[len(prompt):]
 
 
 def test_bfloat16_generation_from_graphs_matches_eager_steps(folders):
