@@ -166,9 +166,10 @@ class RofapelConfig:
         if loop is not None:
             _need(loop, ("start", "stop", "times"), "loop")
             start, stop, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
-            if not (0 <= start < stop <= len(layers)) or times < 1:
-                raise ConfigError("config.json: loop needs 0 <= start < stop <= the number of layers and times >= 1")
-            loop = {"start": start, "stop": stop, "times": times}
+            if not (0 <= start <= stop <= len(layers)) or times < 1:
+                raise ConfigError("config.json: loop needs 0 <= start <= stop <= the number of layers and times >= 1")
+            # an empty range loops over nothing: the layers run once, in order
+            loop = {"start": start, "stop": stop, "times": times} if start < stop else None
         return cls(width=int(raw["width"]), vocab=int(raw["vocab"]), eps=float(raw["norm"]["eps"]),
                    embed_scale=float(raw["embedding"]["scale"]), layers=layers, loop=loop,
                    architecture=str(raw.get("architecture") or "Rofapel"), eos_token_id=raw.get("eos_token_id"),
@@ -273,6 +274,8 @@ def rofapel_spec(config: RofapelConfig) -> ModelSpec:
     sizes = {"vocab_size": config.vocab, "hidden_size": width}
     # a layer without a feed-forward has no use for a second norm: a file that stores one all the same is read
     unused = {f"l{i}.norm2" for i, layer in enumerate(config.layers) if layer.get("mlp") is None}
+    if config.loop is None:
+        unused |= {"loop.in", "loop.step"}     # of a loop over an empty range
     return ModelSpec(
         hidden_size=width, vocab_size=config.vocab, layers=layers, run=rofapel_run_list(len(layers), config.loop),
         final_norm=norm, tie_word_embeddings=False, position_rows=1,

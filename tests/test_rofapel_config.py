@@ -142,6 +142,11 @@ def test_optional_blocks_may_be_absent():
     assert "l0.mlp.shared.up.weight" not in names and "l1.norm2.weight" not in names and "loop.in.weight" not in names
     assert model.pass_mix is None and model.pass_vectors is None
     assert model.spec.map_name("l1.norm2") is None and model.spec.map_name("l0.norm2") == "l0.norm2.weight"
+    # a loop over an empty range is no loop, and its tensors, if a file has them, are passed over
+    cfg["loop"] = {"start": 2, "stop": 2, "times": 3}
+    model = _spec(cfg)
+    assert [e.layer for e in model.spec.run] == [0, 1, 2] and model.pass_mix is None
+    assert model.spec.map_name("loop.in") is None and model.spec.map_name("loop.step") is None
 
 
 def test_random_weights_folder_loads_back(tmp_path):
